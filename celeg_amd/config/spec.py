@@ -46,6 +46,10 @@ class LayerSpec:
     # norms of the sub-layers' outputs, where the arrangement norms before and after ("sandwich_norm")
     mixer_post_norm: Optional[PartSpec] = None
     ffn_post_norm: Optional[PartSpec] = None
+    # what the rows' token ids add to the stream behind the sub-layers, and how the stream behind
+    # the layer is mixed from the results of all entries of the run order so far
+    token_input: Optional[PartSpec] = None
+    depth_mix: Optional[PartSpec] = None
 
     def to_json(self) -> Dict[str, Any]:
         out = {"mixer": self.mixer.to_json(), "mixer_norm": self.mixer_norm.to_json(),
@@ -59,6 +63,10 @@ class LayerSpec:
             out["mixer_post_norm"] = self.mixer_post_norm.to_json()
         if self.ffn_post_norm is not None:
             out["ffn_post_norm"] = self.ffn_post_norm.to_json()
+        if self.token_input is not None:
+            out["token_input"] = self.token_input.to_json()
+        if self.depth_mix is not None:
+            out["depth_mix"] = self.depth_mix.to_json()
         return out
 
     @classmethod
@@ -67,7 +75,7 @@ class LayerSpec:
         return cls(PartSpec.from_json(l["mixer"]), PartSpec.from_json(l["mixer_norm"]),
                    PartSpec.from_json(l["ffn"]), PartSpec.from_json(l["ffn_norm"]),
                    l.get("arrangement", "pre_norm"), link("mixer_link"), link("ffn_link"),
-                   link("mixer_post_norm"), link("ffn_post_norm"))
+                   link("mixer_post_norm"), link("ffn_post_norm"), link("token_input"), link("depth_mix"))
 
 
 @dataclass(frozen=True)
@@ -128,7 +136,8 @@ class ModelSpec:
         parts = [self.embedding] + ([self.reinjection] if self.reinjection is not None else [])
         for layer in self.layers:
             parts += [layer.mixer_norm, layer.mixer, layer.ffn_norm, layer.ffn]
-            parts += [p for p in (layer.mixer_link, layer.ffn_link, layer.mixer_post_norm, layer.ffn_post_norm)
+            parts += [p for p in (layer.mixer_link, layer.ffn_link, layer.mixer_post_norm, layer.ffn_post_norm,
+                                       layer.token_input, layer.depth_mix)
                       if p is not None]
         parts += [self.final_norm, self.head]
         return parts

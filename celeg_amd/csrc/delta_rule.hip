@@ -52,9 +52,10 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_prepare_kernel(
     if (unit == 2 * G + H) {
         for (int h = lane; h < H; h += CELEG_WAVE) {
             const float b = to_float(proj[static_cast<size_t>(t) * ld + col_b + h]);
-            const float a = to_float(proj[static_cast<size_t>(t) * ld + col_a + h]);
+            const float a = a_log ? to_float(proj[static_cast<size_t>(t) * ld + col_a + h]) : 0.f;
             beta_decay[static_cast<size_t>(t) * 2 * H + h] = dr_sigmoid(b);
-            beta_decay[static_cast<size_t>(t) * 2 * H + H + h] = expf(-expf(a_log[h]) * dr_softplus(a + dt_bias[h]));
+            // (a_log null: the decay is made elsewhere, per key channel)
+            if (a_log) beta_decay[static_cast<size_t>(t) * 2 * H + H + h] = expf(-expf(a_log[h]) * dr_softplus(a + dt_bias[h]));
         }
         return;
     }
@@ -379,11 +380,11 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_scan_reg_kernel(
         for (int i = 0; i < DPL; ++i) mine[static_cast<size_t>(sub * DPL + i) * V + j] = S[i];
 }
 
-// one wavefront per (row, head): out = o / sqrt(mean(o^2) + eps) * w * silu(gate)
+// one wavefront per (row, head): out = o / sqrt(mean(o^2) + eps) * w * act(gate), act silu (0) or sigmoid (1)
 template <typename T>
 __global__ __launch_bounds__(CELEG_WAVE) void delta_gated_norm_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                                                       const T* __restrict__ gate, int ldg, float eps,
-                                                                      T* __restrict__ out, int H, int V) {
+                                                                      T* __restrict__ out, int H, int V, int act) {
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const float* row = o + (static_cast<size_t>(t) * H + h) * V;
     float sum = 0.f;
@@ -392,7 +393,7 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_gated_norm_kernel(const floa
     const float inv = 1.0f / sqrtf(sum / static_cast<float>(V) + eps);
     for (int j = lane; j < V; j += CELEG_WAVE) {
         const float z = to_float(gate[static_cast<size_t>(t) * ldg + h * V + j]);
-        out[(static_cast<size_t>(t) * H + h) * V + j] = from_float<T>(row[j] * inv * w[j] * dr_silu(z));
+        out[(static_cast<size_t>(t) * H + h) * V + j] = from_float<T>(row[j] * inv * w[j] * (act == 1 ? dr_sigmoid(z) : dr_silu(z)));
     }
 }
 
@@ -464,14 +465,14 @@ extern "C" int celeg_delta_scan(const float* qk, const float* v, const float* be
 }
 
 extern "C" int celeg_delta_gated_norm(const float* o, const float* w, const void* gate, int ldg, int dtype, float eps, void* out,
-                                      int n_tokens, int H, int V, hipStream_t stream) {
+                                      int n_tokens, int H, int V, int act, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     dim3 grid(n_tokens, H), block(CELEG_WAVE);
     if (dtype == CELEG_F32)
         hipLaunchKernelGGL(delta_gated_norm_kernel<float>, grid, block, 0, stream, o, w, static_cast<const float*>(gate), ldg, eps,
-                           static_cast<float*>(out), H, V);
+                           static_cast<float*>(out), H, V, act);
     else
         hipLaunchKernelGGL(delta_gated_norm_kernel<bf16>, grid, block, 0, stream, o, w, static_cast<const bf16*>(gate), ldg, eps,
-                           static_cast<bf16*>(out), H, V);
+                           static_cast<bf16*>(out), H, V, act);
     return CELEG_LAUNCH_RESULT();
 }

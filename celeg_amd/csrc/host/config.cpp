@@ -818,6 +818,249 @@ ModelSpec kifetar_build_spec(const Json& c) {
 
 }  // namespace
 
+// ---------------------------------------------------------------------------- Kivorax
+// A decoder whose layers read one norm for both sub-layers (x += mixer(norm(x)) + ff(norm(x))),
+// add a gated row of a per-layer token table behind them, and hand on a weighted sum of the
+// results of all layers so far.  config.json describes every layer by itself:
+//   {"architecture": "Kivorax", "vocab", "width", "norm": {"eps"}, "embedding": {"scale"} (absent: 1),
+//    "token_side": {"dim"} (absent: no token input), "max_context" (an engine limit; optional),
+//    "layers": [{"type": "parallel",
+//                "mixer": {"left": {"heads", "kv_heads", "dim", "vdim", "scale", "q_temp": {"coef", "every"} (optional)},
+//                          "right": {"width", "blocks", "conv"}},
+//                "mlp": null | {"kind": "dense", "ff"} | {"kind": "moe", "expert": {"ff"}, "router": {"experts", "top"}}},
+//               {"type": "channel_delta", "mixer": {"heads", "kv_heads", "dim", "vdim", "conv"}, "mlp": ...},
+//               {"type": "gla", "mixer": {"heads", "dim", "vdim", "tau"}, "mlp": ...}]}
+// The widths of the two-step projections (a1/a2 of the decays, g1/g2 of the delta rule's gate) are the
+// checkpoint's ("decay_rank" / "gate_rank" of a mixer where no checkpoint is at hand, else 16); a layer
+// mixes over depth where the checkpoint holds its "dwa" (without a checkpoint: every layer does).
+// Tensors: embed, side.embed, final.norm, head, l<i>.norm1, l<i>.dwa, l<i>.side.{gate,proj,norm},
+// parallel: l<i>.mix.left.{q,k,v,r1,r2,g,o,out}, l<i>.mix.right.{y,y.b,x,x.b,conv,conv.b,ra,ra.b,ri,ri.b,lam,o,out};
+// channel_delta: l<i>.mix.{q,q.conv,k,k.conv,v,v.conv,b,A_log,dt_bias,a1,a2,g1,g2,norm,o};
+// gla: l<i>.mix.{q,k,v,g,a1,a2,a2.b,norm,o}; l<i>.mlp.{up,up.b,down,down.b} or l<i>.mlp.router, l<i>.mlp.e<j>.{up,down}.
+namespace {
+
+// the number of rows of a checkpoint's tensor, or of the mixer's own key, or 16
+long long kivorax_rank(const TensorShapes* shapes, const std::string& tensor, const Json& mixer, const char* key,
+                       const std::string& where) {
+    if (shapes) {
+        auto it = shapes->find(tensor);
+        if (it != shapes->end() && !it->second.empty() && it->second[0] > 0) return it->second[0];
+    }
+    if (!mixer[key].is_null()) return regipel_int(mixer, key, where);
+    return 16;
+}
+
+Json kivorax_read_config(const Json& raw, const TensorShapes* shapes) {
+    if (!raw.is_object()) throw ConfigError("config.json is not an object");
+    Json out = Json::object();
+    out.set("architecture", "Kivorax");
+    out.set("vocab", regipel_int(raw, "vocab", ""));
+    const long long width = regipel_int(raw, "width", "");
+    out.set("width", width);
+    const double eps = regipel_number(regipel_object(raw, "norm", ""), "eps", "norm.");
+    if (!(eps > 0)) throw ConfigError("config.json: 'norm.eps' must be positive");
+    out.set("norm", Json::object().set("eps", eps));
+    double embedding_scale = 1.0;
+    if (!raw["embedding"].is_null()) embedding_scale = regipel_number(regipel_object(raw, "embedding", ""), "scale", "embedding.");
+    out.set("embedding", Json::object().set("scale", embedding_scale));
+    out.set("token_side", raw["token_side"].is_null()
+                              ? Json()
+                              : Json::object().set("dim", regipel_int(regipel_object(raw, "token_side", ""), "dim", "token_side.")));
+    out.set("max_context", raw["max_context"].is_null() ? 131072LL : regipel_int(raw, "max_context", ""));
+    if (!raw["layers"].is_array() || raw["layers"].size() == 0) throw ConfigError("config.json: 'layers' must be a list of layers");
+    Json layers = Json::array();
+    int i = 0;
+    for (const Json& l : raw["layers"].items()) {
+        const std::string prefix = "l" + std::to_string(i) + ".";
+        const std::string where = "layers[" + std::to_string(i++) + "].";
+        if (!l.is_object()) throw ConfigError("config.json: " + where + " must be an object");
+        const std::string type = l.get_string("type", "");
+        const Json& m = regipel_object(l, "mixer", where);
+        const std::string mw = where + "mixer.";
+        Json mixer = Json::object();
+        if (type == "parallel") {
+            const Json& a = regipel_object(m, "left", mw);
+            const std::string aw = mw + "left.";
+            const long long heads = regipel_int(a, "heads", aw), kv_heads = regipel_int(a, "kv_heads", aw);
+            if (heads % kv_heads) throw ConfigError("config.json: " + aw + "'heads' must be a multiple of 'kv_heads'");
+            Json left = Json::object().set("heads", heads).set("kv_heads", kv_heads).set("dim", regipel_int(a, "dim", aw))
+                            .set("vdim", regipel_int(a, "vdim", aw)).set("scale", regipel_number(a, "scale", aw));
+            if (left["vdim"].as_int() > 256) throw ConfigError("config.json: " + aw + "'vdim' may be at most 256");
+            Json q_temp;
+            if (!a["q_temp"].is_null()) {
+                const Json& qt = regipel_object(a, "q_temp", aw);
+                q_temp = Json::object().set("coef", regipel_number(qt, "coef", aw + "q_temp.")).set("every", regipel_int(qt, "every", aw + "q_temp."));
+            }
+            left.set("q_temp", q_temp);
+            const Json& r = regipel_object(m, "right", mw);
+            const std::string rw = mw + "right.";
+            const long long inner = regipel_int(r, "width", rw), blocks = regipel_int(r, "blocks", rw);
+            if (inner % blocks) throw ConfigError("config.json: " + rw + "'width' must be a multiple of 'blocks'");
+            Json right = Json::object().set("width", inner).set("blocks", blocks).set("conv", regipel_int(r, "conv", rw));
+            mixer.set("left", left).set("right", right);
+        } else if (type == "channel_delta") {
+            const long long heads = regipel_int(m, "heads", mw), kv_heads = regipel_int(m, "kv_heads", mw);
+            if (heads % kv_heads) throw ConfigError("config.json: " + mw + "'heads' must be a multiple of 'kv_heads'");
+            mixer.set("heads", heads).set("kv_heads", kv_heads).set("dim", regipel_int(m, "dim", mw)).set("vdim", regipel_int(m, "vdim", mw))
+                .set("conv", regipel_int(m, "conv", mw))
+                .set("decay_rank", kivorax_rank(shapes, prefix + "mix.a1", m, "decay_rank", mw))
+                .set("gate_rank", kivorax_rank(shapes, prefix + "mix.g1", m, "gate_rank", mw));
+            if (mixer["dim"].as_int() > 256) throw ConfigError("config.json: " + mw + "'dim' may be at most 256");
+        } else if (type == "gla") {
+            mixer.set("heads", regipel_int(m, "heads", mw)).set("dim", regipel_int(m, "dim", mw)).set("vdim", regipel_int(m, "vdim", mw))
+                .set("tau", regipel_number(m, "tau", mw)).set("decay_rank", kivorax_rank(shapes, prefix + "mix.a1", m, "decay_rank", mw));
+            if (!(mixer["tau"].as_double() > 0)) throw ConfigError("config.json: " + mw + "'tau' must be positive");
+            if (mixer["dim"].as_int() > 256) throw ConfigError("config.json: " + mw + "'dim' may be at most 256");
+        } else {
+            throw ConfigError("config.json: " + where + "'type' is '" + type + "'; known types are ['parallel', 'channel_delta', 'gla']");
+        }
+        Json mlp;
+        if (!l["mlp"].is_null()) {
+            const Json& f = regipel_object(l, "mlp", where);
+            const std::string fw = where + "mlp.";
+            const std::string kind = f.get_string("kind", "");
+            if (kind == "dense") {
+                mlp = Json::object().set("kind", kind).set("ff", regipel_int(f, "ff", fw));
+            } else if (kind == "moe") {
+                const Json& router = regipel_object(f, "router", fw);
+                const long long experts = regipel_int(router, "experts", fw + "router."), top = regipel_int(router, "top", fw + "router.");
+                if (top > experts) throw ConfigError("config.json: " + fw + "'router.top' exceeds 'router.experts'");
+                if (experts > 512) throw ConfigError("config.json: " + fw + "'router.experts' may be at most 512");
+                mlp = Json::object().set("kind", kind)
+                          .set("expert", Json::object().set("ff", regipel_int(regipel_object(f, "expert", fw), "ff", fw + "expert.")))
+                          .set("router", Json::object().set("experts", experts).set("top", top));
+            } else {
+                throw ConfigError("config.json: " + fw + "'kind' is '" + kind + "'; known kinds are ['dense', 'moe']");
+            }
+        }
+        const bool depth = shapes ? shapes->count(prefix + "dwa") > 0 : l.get_bool("depth_average", true);
+        layers.push(Json::object().set("type", type).set("mixer", mixer).set("mlp", mlp).set("depth_average", depth));
+    }
+    out.set("layers", layers);
+    for (const char* key : {"bos_token_id", "eos_token_id"})
+        if (!raw[key].is_null()) out.set(key, raw[key]);
+    return out;
+}
+
+ModelSpec kivorax_build_spec(const Json& c) {
+    const long long W = c["width"].as_int();
+    const double eps = c["norm"]["eps"].as_double();
+    const long long n_layers = static_cast<long long>(c["layers"].size());
+    auto norm = [&](const std::string& name) {
+        PartSpec p;
+        p.kind = "rmsnorm";
+        p.params = Json::object().set("width", W).set("eps", eps);
+        p.tensors = {{"weight", name}};
+        return p;
+    };
+    ModelSpec spec;
+    int i = 0;
+    for (const Json& l : c["layers"].items()) {
+        const std::string p = "l" + std::to_string(i) + ".";
+        const Json& m = l["mixer"];
+        const std::string type = l["type"].as_string();
+        LayerSpec layer;
+        layer.arrangement = "parallel";
+        if (type == "parallel") {
+            const Json& a = m["left"];
+            const Json& r = m["right"];
+            PartSpec left, right;
+            left.kind = "biased_attention";
+            left.params = Json::object().set("width", W).set("heads", a["heads"]).set("kv_heads", a["kv_heads"]).set("head_dim", a["dim"])
+                              .set("v_dim", a["vdim"]).set("scale", a["scale"]).set("distance_bias", true).set("gate", "sigmoid");
+            if (!a["q_temp"].is_null()) left.params.set("query_temperature", a["q_temp"]);
+            right.kind = "linear_recurrent_unit";
+            right.params = Json::object().set("width", W).set("inner", r["width"]).set("blocks", r["blocks"]).set("taps", r["conv"])
+                               .set("decay_scale", 8.0);
+            layer.mixer.kind = "normed_pair";
+            layer.mixer.params = Json::object().set("width", W).set("eps", eps).set("factor", 0.5).set("left", left.to_json())
+                                     .set("right", right.to_json());
+            const std::string lp = p + "mix.left.", rp = p + "mix.right.";
+            layer.mixer.tensors = {{"left_out", lp + "out"}, {"right_out", rp + "out"},
+                                   {"left.q", lp + "q"},     {"left.k", lp + "k"},   {"left.v", lp + "v"},   {"left.o", lp + "o"},
+                                   {"left.r1", lp + "r1"},   {"left.r2", lp + "r2"}, {"left.g", lp + "g"},
+                                   {"right.y", rp + "y"},    {"right.y_bias", rp + "y.b"}, {"right.x", rp + "x"}, {"right.x_bias", rp + "x.b"},
+                                   {"right.conv", rp + "conv"}, {"right.conv_bias", rp + "conv.b"}, {"right.ra", rp + "ra"},
+                                   {"right.ra_bias", rp + "ra.b"}, {"right.ri", rp + "ri"}, {"right.ri_bias", rp + "ri.b"},
+                                   {"right.lam", rp + "lam"}, {"right.o", rp + "o"}};
+        } else if (type == "channel_delta") {
+            layer.mixer.kind = "gated_delta_rule";
+            layer.mixer.params = Json::object().set("width", W).set("heads", m["heads"]).set("kv_heads", m["kv_heads"]).set("dim", m["dim"])
+                                     .set("vdim", m["vdim"]).set("taps", m["conv"]).set("eps", eps).set("decay", "channel")
+                                     .set("decay_rank", m["decay_rank"]).set("gate", "sigmoid").set("gate_rank", m["gate_rank"]);
+            layer.mixer.tensors = {{"q", p + "mix.q"},     {"k", p + "mix.k"},     {"v", p + "mix.v"},   {"q_conv", p + "mix.q.conv"},
+                                   {"k_conv", p + "mix.k.conv"}, {"v_conv", p + "mix.v.conv"}, {"b", p + "mix.b"}, {"A_log", p + "mix.A_log"},
+                                   {"dt_bias", p + "mix.dt_bias"}, {"a1", p + "mix.a1"}, {"a2", p + "mix.a2"}, {"g1", p + "mix.g1"},
+                                   {"g2", p + "mix.g2"},   {"norm", p + "mix.norm"}, {"o", p + "mix.o"}};
+        } else {
+            layer.mixer.kind = "gated_linear_attention";
+            layer.mixer.params = Json::object().set("width", W).set("heads", m["heads"]).set("dim", m["dim"]).set("vdim", m["vdim"])
+                                     .set("tau", m["tau"]).set("decay_rank", m["decay_rank"]).set("eps", eps);
+            layer.mixer.tensors = {{"q", p + "mix.q"},   {"k", p + "mix.k"},   {"v", p + "mix.v"},       {"g", p + "mix.g"},
+                                   {"a1", p + "mix.a1"}, {"a2", p + "mix.a2"}, {"a2_bias", p + "mix.a2.b"}, {"norm", p + "mix.norm"},
+                                   {"o", p + "mix.o"}};
+        }
+        layer.mixer_norm = norm(p + "norm1");
+        layer.ffn_norm.kind = "identity";
+        if (l["mlp"].is_null()) {
+            layer.ffn.kind = "none";
+        } else if (l["mlp"]["kind"].as_string() == "dense") {
+            layer.ffn.kind = "mlp";
+            layer.ffn.params = Json::object().set("width", W).set("ff", l["mlp"]["ff"]).set("activation", "gelu_tanh").set("bias", true);
+            layer.ffn.tensors = {{"up", p + "mlp.up"}, {"up_bias", p + "mlp.up.b"}, {"down", p + "mlp.down"}, {"down_bias", p + "mlp.down.b"}};
+        } else {
+            const Json& f = l["mlp"];
+            const long long experts = f["router"]["experts"].as_int();
+            layer.ffn.kind = "routed_experts";
+            layer.ffn.params = Json::object().set("width", W).set("ff", f["expert"]["ff"]).set("experts", experts)
+                                   .set("top", f["router"]["top"]).set("score", "softmax").set("renormalize", false)
+                                   .set("weight_on", "output").set("gated", false).set("activation", "relu2");
+            layer.ffn.tensors = {{"router", p + "mlp.router"}};
+            for (long long e = 0; e < experts; ++e) {
+                const std::string ep = p + "mlp.e" + std::to_string(e) + ".", n = std::to_string(e);
+                layer.ffn.tensors.emplace_back("up." + n, ep + "up");
+                layer.ffn.tensors.emplace_back("down." + n, ep + "down");
+            }
+        }
+        if (!c["token_side"].is_null()) {
+            const long long dim = c["token_side"]["dim"].as_int();
+            layer.token_input.kind = "gated_table";
+            layer.token_input.params = Json::object().set("width", W).set("vocab", c["vocab"]).set("dim", dim).set("offset", dim * i)
+                                           .set("table_width", dim * n_layers).set("eps", eps);
+            layer.token_input.tensors = {{"table", "side.embed"}, {"gate", p + "side.gate"}, {"proj", p + "side.proj"},
+                                         {"norm", p + "side.norm"}};
+        }
+        if (l["depth_average"].as_bool()) {
+            layer.depth_mix.kind = "weighted_history";
+            layer.depth_mix.params = Json::object().set("entries", static_cast<long long>(i) + 2);
+            layer.depth_mix.tensors = {{"weights", p + "dwa"}};
+        }
+        spec.layers.push_back(std::move(layer));
+        spec.order.push_back(RunStep{i, {}, false});
+        ++i;
+    }
+    spec.architecture = "Kivorax";
+    spec.vocab_size = static_cast<int>(c["vocab"].as_int());
+    spec.hidden_size = static_cast<int>(W);
+    spec.max_context = static_cast<int>(c["max_context"].as_int());
+    spec.embedding.kind = "embedding";
+    spec.embedding.params = Json::object().set("vocab", c["vocab"]).set("width", W).set("scale", c["embedding"]["scale"]);
+    spec.embedding.tensors = {{"table", "embed"}};
+    spec.head.kind = "linear_head";
+    spec.head.params = Json::object().set("vocab", c["vocab"]).set("width", W);
+    spec.head.tensors = {{"weight", "head"}};
+    spec.final_norm = norm("final.norm");
+    if (c["eos_token_id"].is_array())
+        for (const Json& e : c["eos_token_id"].items()) spec.eos_token_ids.push_back(static_cast<int>(e.as_int()));
+    else if (c["eos_token_id"].is_int())
+        spec.eos_token_ids.push_back(static_cast<int>(c["eos_token_id"].as_int()));
+    if (c["bos_token_id"].is_int()) spec.bos_token_id = static_cast<int>(c["bos_token_id"].as_int());
+    spec.validate();
+    return spec;
+}
+
+}  // namespace
+
 namespace {
 void register_builtin() {
     Architecture lfm2;
@@ -842,6 +1085,13 @@ void register_builtin() {
     kifetar.build_spec = kifetar_build_spec;
     table()["Kifetar"] = kifetar;
     table()["kifetar"] = kifetar;
+    Architecture kivorax;
+    kivorax.name = "Kivorax";
+    kivorax.aliases = {"kivorax"};
+    kivorax.read_config = kivorax_read_config;
+    kivorax.build_spec = kivorax_build_spec;
+    table()["Kivorax"] = kivorax;
+    table()["kivorax"] = kivorax;
 }
 
 }  // namespace

@@ -64,7 +64,7 @@ int celeg_moe_plan(const int* ids, int n, int experts, int tile_rows, int* offse
                    int* tile_row0, int* n_tiles, hipStream_t stream);
 int celeg_moe_gather(const void* x, int dtype, const int* entry_at, const float* weights, void* a, int n, int top, int width,
                      hipStream_t stream);
-int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated, const int* offsets,
+int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated, int act, const int* offsets,
                       const int* tile_expert, const int* tile_row0, const int* n_tiles, int max_tiles, int tile_rows, int wide,
                       hipStream_t stream);
 int celeg_moe_combine(const void* y, int dtype, const int* place_of, const float* weights, void* out, int rows, int top,
@@ -169,5 +169,39 @@ int celeg_delta_scan(const float* qk, const float* v, const float* beta_decay, f
                      const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D, int V,
                      int general, const int* token_seq, float* pairs, int n_tokens, hipStream_t stream);
 int celeg_delta_gated_norm(const float* o, const float* w, const void* gate, int ldg, int dtype, float eps, void* out,
-                           int n_tokens, int H, int V, hipStream_t stream);
+                           int n_tokens, int H, int V, int act, hipStream_t stream);
+// layer_glue.hip
+int celeg_activation_bias(const void* x, int ldx, const float* bias, void* out, int ldo, int dtype, int rows, int cols, int act,
+                          hipStream_t stream);
+int celeg_residual_sum(float* h, const void* a, int lda, const void* b, int ldb, void* copy, int dtype, int rows, int width,
+                       hipStream_t stream);
+int celeg_token_gate(const void* z, int ldz, const void* table, int ld_table, int offset, const int* token_ids, void* g, int dtype,
+                     int rows, int dim, hipStream_t stream);
+int celeg_normed_mean(const void* a, int lda, const float* wa, const void* b, int ldb, const float* wb, float eps, float factor,
+                      void* out, int dtype, int rows, int width, hipStream_t stream);
+int celeg_depth_mix(float* history, size_t entry_stride, float* h, const float* w, int n, int rows, int width, hipStream_t stream);
+// biased_attention.hip
+int celeg_kv_store(const void* k, int ldk, const void* v, int ldv, int dtype, void* k_pool, void* v_pool, const int* table,
+                   int table_stride, const int* token_slot, const int* positions, int n_tokens, int kv_heads, int head_dim, int v_dim,
+                   int page_tokens, int n_layers, int layer, hipStream_t stream);
+int celeg_biased_attention(const void* q, int ldq, int dtype, const void* k_pool, const void* v_pool, const int* table,
+                           int table_stride, const int* token_slot, const int* positions, const float* r1, const float* r2,
+                           const void* gate, int ldg, void* out, int ldo, int n_tokens, int q_heads, int kv_heads, int head_dim,
+                           int v_dim, int page_tokens, int n_layers, int layer, float scale, float coef, int every, int window,
+                           hipStream_t stream);
+// linear_scan.hip
+int celeg_lru_gates(const void* x, int ldx, int dtype, const float* conv_w, const float* conv_b, const float* ra_t, const float* ra_b,
+                    const float* ri_t, const float* ri_b, const float* lam, const float* conv_state, size_t state_stride,
+                    const int* positions, const int* token_seq, const int* seq_start, const int* token_slot, float* decay,
+                    float* input, int n_tokens, int width, int blocks, int taps, float decay_scale, hipStream_t stream);
+int celeg_lru_scan(const float* decay, const float* input, const void* y, int ldy, int dtype, float* state, size_t state_stride,
+                   const int* cu_seqlens, const int* seq_slot, void* out, int ldo, int n_seqs, int width, hipStream_t stream);
+int celeg_channel_decay(const void* z, int ldz, int dtype, const float* a_log, const float* dt_bias, float* decay, int n_tokens,
+                        int heads, int dim, hipStream_t stream);
+int celeg_gla_prepare(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const void* z, int ldz, int dtype,
+                      const float* z_bias, float inv_tau, float q_scale, float* qk, float* v32, float* decay, int n_tokens,
+                      int qk_cols, int v_cols, hipStream_t stream);
+int celeg_channel_scan(const float* qk, const float* v, const float* decay, const float* beta, int ld_beta, float* state,
+                       size_t state_stride, const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D,
+                       int V, hipStream_t stream);
 }

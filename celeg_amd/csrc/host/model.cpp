@@ -24,6 +24,25 @@ Model::Model(ModelSpec s) : spec(std::move(s)) {
             throw SpecError("layer " + std::to_string(blocks_.size() - 1) + " ('" + layer.arrangement + "') works on " +
                             std::to_string(blocks_.back()->streams()) + " residual stream(s), the model keeps " +
                             std::to_string(spec.streams));
+        token_inputs_.push_back(layer.token_input.kind.empty() ? nullptr : build_as<TokenInput>("token_input", layer.token_input));
+        depth_mixes_.push_back(layer.depth_mix.kind.empty() ? nullptr : build_as<DepthMix>("depth_mix", layer.depth_mix));
+        if ((token_inputs_.back() || depth_mixes_.back()) && spec.streams != 1)
+            throw SpecError("a token input or a mixture over depth works on one residual stream");
+    }
+    // a mixture over depth reads the results of all entries before its own: its size is fixed by its place
+    for (size_t l = 0; l < depth_mixes_.size(); ++l) {
+        if (!depth_mixes_[l]) continue;
+        int at = -1, times = 0;
+        for (size_t i = 0; i < spec.order.size(); ++i)
+            if (spec.order[i].layer == static_cast<int>(l)) {
+                at = static_cast<int>(i);
+                ++times;
+            }
+        if (times > 1) throw SpecError("layer " + std::to_string(l) + " mixes over depth and runs more than once");
+        if (times == 1 && depth_mixes_[l]->entries() != at + 2)
+            throw SpecError("layer " + std::to_string(l) + " is entry " + std::to_string(at) + " of the run order and mixes " +
+                            std::to_string(depth_mixes_[l]->entries()) + " results, not " + std::to_string(at + 2));
+        if (times == 1) history_entries_ = std::max(history_entries_, at + 2);
     }
     final_norm_ = build_as<Norm>("norm", spec.final_norm);
     head_ = build_as<Head>("head", spec.head);
@@ -67,8 +86,11 @@ void Model::resolve_cache_sharing() {
 std::vector<std::pair<std::string, Part*>> Model::named_parts() {
     std::vector<std::pair<std::string, Part*>> out{{"embedding", embedding_.get()}};
     if (reinjection_) out.emplace_back("reinjection", reinjection_.get());
-    for (size_t i = 0; i < blocks_.size(); ++i)
+    for (size_t i = 0; i < blocks_.size(); ++i) {
         for (const auto& p : blocks_[i]->parts()) out.emplace_back("layers." + std::to_string(i) + "." + p.first, p.second);
+        if (token_inputs_[i]) out.emplace_back("layers." + std::to_string(i) + ".token_input", token_inputs_[i].get());
+        if (depth_mixes_[i]) out.emplace_back("layers." + std::to_string(i) + ".depth_mix", depth_mixes_[i].get());
+    }
     out.emplace_back("final_norm", final_norm_.get());
     out.emplace_back("head", head_.get());
     return out;
@@ -179,7 +201,18 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
         x0 = rt.ws.buf("embedding_rows", DType::F32, {T, width});
         rt.ops.cast(h, x0);
     }
+    // the results of the entries so far (the embedding's rows first), for layers that mix over depth
+    Tensor history;
+    auto history_entry = [&](long long j) {
+        return Tensor::make(history.as<float>() + static_cast<size_t>(j) * static_cast<size_t>(T * width), DType::F32, {T, width});
+    };
+    if (history_entries_ > 0) {
+        history = rt.ws.buf("depth_history", DType::F32, {history_entries_, T, width});
+        rt.ops.cast(h, history_entry(0));
+    }
     for (size_t i = 0; i < spec.order.size(); ++i) {
+        const size_t layer = static_cast<size_t>(spec.order[i].layer);
+        rt.stream_copy = Tensor();
         if (spec.order[i].reinject) {
             if (delta.defined()) rt.ops.norm_step(h, &delta, nullptr, nullptr, nullptr);     // the pending sum first
             delta = Tensor();
@@ -188,7 +221,28 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
             reinjection_->forward(h, x0, rt);
             rt.mark("reinjection");
         }
-        delta = blocks_[static_cast<size_t>(spec.order[i].layer)]->forward(hs, delta, batch, caches_[i], rt);
+        delta = blocks_[layer]->forward(hs, delta, batch, caches_[i], rt);
+        if (token_inputs_[layer] || depth_mixes_[layer] || (history.defined() && static_cast<int>(i) + 1 < history_entries_)) {
+            if (delta.defined()) rt.ops.norm_step(h, &delta, nullptr, nullptr, nullptr);     // the pending sum first
+            if (delta.defined()) rt.stream_copy = Tensor();
+            delta = Tensor();
+            rt.stream_stat_blocks = 0;
+            rt.stream_has_bf16 = false;
+            if (token_inputs_[layer]) {
+                if (!rt.stream_copy.defined()) {
+                    rt.stream_copy = rt.ws.buf("stream_copy", rt.dtype, {T, width});
+                    rt.ops.cast(h, rt.stream_copy);
+                }
+                token_inputs_[layer]->forward(h, rt.stream_copy, batch, rt);
+                rt.mark("token input");
+            }
+            if (depth_mixes_[layer]) {
+                depth_mixes_[layer]->forward(history, h, rt);
+                rt.mark("depth mix");
+            } else if (history.defined() && static_cast<int>(i) + 1 < history_entries_) {
+                rt.ops.cast(h, history_entry(static_cast<long long>(i) + 1));
+            }
+        }
         if (rt.after_layer) {
             if (S > 1) rt.ops.streams_sum(hs, h, S);
             rt.after_layer(static_cast<int>(i), h, delta.defined() ? &delta : nullptr);

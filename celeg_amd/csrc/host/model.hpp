@@ -45,6 +45,10 @@ private:
     std::unique_ptr<Embedding> embedding_;
     std::unique_ptr<Reinjection> reinjection_;
     std::vector<std::unique_ptr<Block>> blocks_;
+    // per layer, or null: what the rows' token ids add behind the layer, how the stream behind it is mixed over depth
+    std::vector<std::unique_ptr<TokenInput>> token_inputs_;
+    std::vector<std::unique_ptr<DepthMix>> depth_mixes_;
+    int history_entries_ = 0;      // results a step keeps for the depth mixes (0: none)
     std::unique_ptr<Norm> final_norm_;
     std::unique_ptr<Head> head_;
     std::vector<LayerCache> caches_;

@@ -58,6 +58,10 @@ const char* path_name(Path p) {
         case Path::AttentionLatent: return "attention_latent";
         case Path::AttentionLatentRows: return "attention_latent_rows";
         case Path::AttentionLatentDecode: return "attention_latent_decode";
+        case Path::AttentionBiased: return "attention_biased";
+        case Path::AttentionBiasedRows: return "attention_biased_rows";
+        case Path::ChannelScan: return "channel_scan";
+        case Path::LinearRecurrentUnit: return "linear_recurrent_unit";
         case Path::RoutedExperts: return "routed_experts";
         case Path::LinearF32: return "linear_f32";
         case Path::LinearLibrary: return "linear_library";
@@ -334,7 +338,8 @@ void Ops::moe_gather(const Tensor& x, const RoutePlan& p, bool weighted, const T
                                   p.n, p.top, static_cast<int>(x.shape[1]), stream), "moe_gather");
 }
 
-void Ops::moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool gated, const RoutePlan& p) {
+void Ops::moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool gated, const RoutePlan& p, int act) {
+    need(act == 0 || (act == 1 && !gated), "moe_product: act is 0, or 1 (square of relu) where the product is not gated");
     dev(a, "a");
     dev(w, "w", a.dtype);
     dev(out, "out", a.dtype);
@@ -345,7 +350,7 @@ void Ops::moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool 
     need(p.tile_rows == celeg_moe_tile_rows(0) || moe_matrix_cores_ok(a.dtype, out.shape[1], a.shape[1]),
          "moe_product: the plan was made for the matrix cores, which do not take this product");
     kernel_check(celeg_moe_product(a.data, w.data, out.data, dt(a, "a"), static_cast<int>(out.shape[1]),
-                                   static_cast<int>(a.shape[1]), gated ? 1 : 0, p.offsets.as<int>(), p.tile_expert.as<int>(),
+                                   static_cast<int>(a.shape[1]), gated ? 1 : 0, act, p.offsets.as<int>(), p.tile_expert.as<int>(),
                                    p.tile_row0.as<int>(), p.n_tiles.as<int>(), p.max_tiles, p.tile_rows,
                                    p.n >= 8 * p.experts ? 1 : 0, stream), "moe_product");
 }
@@ -794,13 +799,17 @@ void Ops::delta_prepare(const Tensor& proj, int col_b, int col_a, const DeltaSha
     const long long T = proj.shape[0], qkw = 2LL * s.kv_heads * s.dim, vw = static_cast<long long>(s.heads) * s.vdim, C = qkw + vw;
     need(s.heads > 0 && s.kv_heads > 0 && s.heads % s.kv_heads == 0 && s.dim > 0 && s.vdim > 0 && s.taps >= 1,
          "delta_prepare: heads must be a positive multiple of kv_heads, sizes positive");
+    if (!a_log.defined()) col_a = col_b;
     need(proj.ndim == 2 && T == batch.n_tokens && col_b >= C && col_a >= C && col_b + s.heads <= proj.shape[1] &&
              col_a + s.heads <= proj.shape[1], "delta_prepare: the projections' columns do not fit");
     dev(conv_w, "conv_w", DType::F32);
     need(conv_w.numel() == C * s.taps, "delta_prepare: one row of taps per channel");
-    dev(a_log, "a_log", DType::F32);
-    dev(dt_bias, "dt_bias", DType::F32);
-    need(a_log.numel() == s.heads && dt_bias.numel() == s.heads, "delta_prepare: one decay constant and bias per head");
+    // (a_log undefined: no decay per head is made; the second half of beta_decay is left alone)
+    if (a_log.defined()) {
+        dev(a_log, "a_log", DType::F32);
+        dev(dt_bias, "dt_bias", DType::F32);
+        need(a_log.numel() == s.heads && dt_bias.numel() == s.heads, "delta_prepare: one decay constant and bias per head");
+    }
     dev(conv_state, "conv_state", DType::F32, false);
     need(conv_state.ndim == 3 && conv_state.shape[1] == std::max(s.taps - 1, 1) && conv_state.shape[2] == C &&
              conv_state.stride[2] == 1 && conv_state.stride[1] == C, "delta_prepare: saved inputs must be [slots, taps - 1, channels]");
@@ -810,8 +819,8 @@ void Ops::delta_prepare(const Tensor& proj, int col_b, int col_a, const DeltaSha
     need(qk.numel() == T * qkw && v.numel() == T * vw && beta_decay.numel() == T * 2 * s.heads, "delta_prepare: outputs do not fit");
     const int ld = rows_of(proj, "proj");
     took(Path::DeltaRule);
-    kernel_check(celeg_delta_prepare(proj.data, ld, dt(proj, "proj"), col_b, col_a, conv_w.as<float>(), a_log.as<float>(),
-                                     dt_bias.as<float>(), conv_state.as<float>(), static_cast<size_t>(conv_state.stride[0]),
+    kernel_check(celeg_delta_prepare(proj.data, ld, dt(proj, "proj"), col_b, col_a, conv_w.as<float>(),
+                                     a_log.defined() ? a_log.as<float>() : nullptr, a_log.defined() ? dt_bias.as<float>() : nullptr, conv_state.as<float>(), static_cast<size_t>(conv_state.stride[0]),
                                      batch.positions, batch.token_seq, batch.seq_start, batch.token_slot, qk.as<float>(), v.as<float>(),
                                      beta_decay.as<float>(), static_cast<int>(T), s.kv_heads, s.heads, s.dim, s.vdim, s.taps, stream),
                  "delta_prepare");
@@ -844,7 +853,9 @@ void Ops::delta_scan(const Tensor& qk, const Tensor& v, const Tensor& beta_decay
                  "delta_scan");
 }
 
-void Ops::delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim) {
+void Ops::delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim,
+                           int act) {
+    need(act == 0 || act == 1, "delta_gated_norm: act is 0 (silu) or 1 (sigmoid)");
     dev(o, "o", DType::F32);
     dev(weight, "weight", DType::F32);
     dev(gate, "gate", out.dtype, false);
@@ -853,7 +864,243 @@ void Ops::delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& 
     need(o.ndim == 2 && o.shape[1] == w && out.ndim == 2 && out.shape[0] == T && out.shape[1] == w && out.contiguous() &&
              gate.ndim == 2 && gate.shape[0] == T && gate.shape[1] == w && weight.numel() == vdim, "delta_gated_norm: shapes do not fit");
     kernel_check(celeg_delta_gated_norm(o.as<float>(), weight.as<float>(), gate.data, rows_of(gate, "gate"), dt(out, "out"), eps, out.data,
-                                        static_cast<int>(T), heads, vdim, stream), "delta_gated_norm");
+                                        static_cast<int>(T), heads, vdim, act, stream), "delta_gated_norm");
+}
+
+// ---------------------------------------------------------------------------- states with a decay per key channel
+void Ops::channel_decay(const Tensor& z, const Tensor& a_log, const Tensor& dt_bias, const Tensor& decay, int heads, int dim) {
+    dev(z, "z");
+    dev(a_log, "a_log", DType::F32);
+    dev(dt_bias, "dt_bias", DType::F32);
+    dev(decay, "decay", DType::F32);
+    const long long T = z.shape[0], cols = static_cast<long long>(heads) * dim;
+    need(z.ndim == 2 && z.shape[1] == cols && a_log.numel() == heads && dt_bias.numel() == cols && decay.numel() == T * cols,
+         "channel_decay: z [rows, heads * dim], a_log [heads], dt_bias [heads * dim]");
+    kernel_check(celeg_channel_decay(z.data, rows_of(z, "z"), dt(z, "z"), a_log.as<float>(), dt_bias.as<float>(), decay.as<float>(),
+                                     static_cast<int>(T), heads, dim, stream), "channel_decay");
+}
+
+void Ops::gla_prepare(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& z, const Tensor* z_bias, float tau, float q_scale,
+                      const Tensor& qk, const Tensor& v32, const Tensor& decay) {
+    dev(q, "q");
+    dev(k, "k", q.dtype, false);
+    dev(v, "v", q.dtype, false);
+    dev(z, "z", q.dtype, false);
+    dev(qk, "qk", DType::F32);
+    dev(v32, "v32", DType::F32);
+    dev(decay, "decay", DType::F32);
+    const long long T = q.shape[0], qc = q.shape[1], vc = v.shape[1];
+    need(q.ndim == 2 && k.ndim == 2 && v.ndim == 2 && z.ndim == 2 && k.shape[0] == T && v.shape[0] == T && z.shape[0] == T &&
+             k.shape[1] == qc && z.shape[1] == qc && qk.numel() == T * 2 * qc && v32.numel() == T * vc && decay.numel() == T * qc,
+         "gla_prepare: shapes do not fit");
+    need(tau > 0.f, "gla_prepare: tau must be positive");
+    if (z_bias) {
+        dev(*z_bias, "z_bias", DType::F32);
+        need(z_bias->numel() == qc, "gla_prepare: one bias per decay channel");
+    }
+    kernel_check(celeg_gla_prepare(q.data, rows_of(q, "q"), k.data, rows_of(k, "k"), v.data, rows_of(v, "v"), z.data, rows_of(z, "z"),
+                                   dt(q, "q"), z_bias ? z_bias->as<float>() : nullptr, 1.0f / tau, q_scale, qk.as<float>(),
+                                   v32.as<float>(), decay.as<float>(), static_cast<int>(T), static_cast<int>(qc), static_cast<int>(vc),
+                                   stream), "gla_prepare");
+}
+
+void Ops::channel_scan(const Tensor& qk, const Tensor& v, const Tensor& decay, const float* beta, int beta_ld, const Tensor& state,
+                       const Tensor& out, const DeltaShape& s, const StepBatch& batch) {
+    dev(qk, "qk", DType::F32);
+    dev(v, "v", DType::F32);
+    dev(decay, "decay", DType::F32);
+    dev(out, "out", DType::F32);
+    dev(state, "state", DType::F32, false);
+    need(s.heads > 0 && s.kv_heads > 0 && s.heads % s.kv_heads == 0 && s.dim > 0 && s.vdim > 0,
+         "channel_scan: heads must be a positive multiple of kv_heads, sizes positive");
+    const long long T = batch.n_tokens, per_slot = static_cast<long long>(s.heads) * s.dim * s.vdim;
+    need(qk.numel() == T * 2 * s.kv_heads * s.dim && v.numel() == T * s.heads * s.vdim && out.numel() == v.numel() &&
+             decay.numel() == T * s.heads * s.dim, "channel_scan: rows do not fit");
+    need(state.ndim >= 2 && state.numel() / state.shape[0] == per_slot && state.stride[state.ndim - 1] == 1,
+         "channel_scan: state must be [slots, heads, dim, vdim]");
+    need(s.dim <= 256, "channel_scan: dim " + std::to_string(s.dim) + " exceeds 256");
+    need(!beta || beta_ld >= s.heads, "channel_scan: a row of write strengths holds one per head");
+    took(Path::ChannelScan);
+    kernel_check(celeg_channel_scan(qk.as<float>(), v.as<float>(), decay.as<float>(), beta, beta_ld, state.as<float>(),
+                                    static_cast<size_t>(state.stride[0]), batch.cu_seqlens, batch.seq_slot, out.as<float>(),
+                                    batch.n_seqs, s.kv_heads, s.heads, s.dim, s.vdim, stream), "channel_scan");
+}
+
+// ---------------------------------------------------------------------------- linear recurrent unit
+void Ops::lru_gates(const Tensor& x, const Tensor& conv_w, const Tensor* conv_b, const Tensor& ra_t, const Tensor& ra_b,
+                    const Tensor& ri_t, const Tensor& ri_b, const Tensor& lam, const Tensor& conv_state, const Tensor& decay,
+                    const Tensor& input, const LruShape& s, const StepBatch& batch) {
+    dev(x, "x");
+    need(s.width > 0 && s.blocks > 0 && s.width % s.blocks == 0 && s.taps >= 1, "lru_gates: width must be a positive multiple of blocks");
+    const long long T = x.shape[0], W = s.width, bw = W / s.blocks;
+    need(x.ndim == 2 && x.shape[1] == W && T == batch.n_tokens, "lru_gates: x must be [rows, width]");
+    dev(conv_w, "conv_w", DType::F32);
+    need(conv_w.numel() == W * s.taps, "lru_gates: one row of taps per channel");
+    if (conv_b) {
+        dev(*conv_b, "conv_b", DType::F32);
+        need(conv_b->numel() == W, "lru_gates: one convolution bias per channel");
+    }
+    for (const Tensor* m : {&ra_t, &ri_t}) {
+        dev(*m, "gate matrix", DType::F32);
+        need(m->numel() == s.blocks * bw * bw, "lru_gates: gate matrices are [blocks, width / blocks, width / blocks]");
+    }
+    for (const Tensor* b : {&ra_b, &ri_b, &lam}) {
+        dev(*b, "gate vector", DType::F32);
+        need(b->numel() == W, "lru_gates: gate biases and lam have one entry per channel");
+    }
+    dev(conv_state, "conv_state", DType::F32, false);
+    need(conv_state.ndim == 3 && conv_state.shape[1] == std::max(s.taps - 1, 1) && conv_state.shape[2] == W &&
+             conv_state.stride[2] == 1 && conv_state.stride[1] == W, "lru_gates: saved inputs must be [slots, taps - 1, width]");
+    dev(decay, "decay", DType::F32);
+    dev(input, "input", DType::F32);
+    need(decay.numel() == T * W && input.numel() == T * W, "lru_gates: outputs do not fit");
+    const int ld = rows_of(x, "x");
+    took(Path::LinearRecurrentUnit);
+    kernel_check(celeg_lru_gates(x.data, ld, dt(x, "x"), conv_w.as<float>(), conv_b ? conv_b->as<float>() : nullptr, ra_t.as<float>(),
+                                 ra_b.as<float>(), ri_t.as<float>(), ri_b.as<float>(), lam.as<float>(), conv_state.as<float>(),
+                                 static_cast<size_t>(conv_state.stride[0]), batch.positions, batch.token_seq, batch.seq_start,
+                                 batch.token_slot, decay.as<float>(), input.as<float>(), static_cast<int>(T), s.width, s.blocks, s.taps,
+                                 s.decay_scale, stream), "lru_gates");
+    // (after every row has read the old saved inputs)
+    kernel_check(celeg_delta_conv_state(x.data, ld, dt(x, "x"), conv_state.as<float>(), static_cast<size_t>(conv_state.stride[0]),
+                                        batch.cu_seqlens, batch.seq_slot, batch.n_seqs, s.width, s.taps, stream), "lru_conv_state");
+}
+
+void Ops::lru_scan(const Tensor& decay, const Tensor& input, const Tensor& y, const Tensor& state, const Tensor& out,
+                   const StepBatch& batch) {
+    dev(decay, "decay", DType::F32);
+    dev(input, "input", DType::F32);
+    dev(y, "y");
+    dev(out, "out", y.dtype, false);
+    dev(state, "state", DType::F32, false);
+    const long long T = batch.n_tokens, W = y.shape[1];
+    need(y.ndim == 2 && out.ndim == 2 && y.shape[0] == T && out.shape[0] == T && out.shape[1] == W && decay.numel() == T * W &&
+             input.numel() == T * W, "lru_scan: rows do not fit");
+    need(state.ndim == 2 && state.shape[1] == W && state.stride[1] == 1, "lru_scan: state must be [slots, width]");
+    kernel_check(celeg_lru_scan(decay.as<float>(), input.as<float>(), y.data, rows_of(y, "y"), dt(y, "y"), state.as<float>(),
+                                static_cast<size_t>(state.stride[0]), batch.cu_seqlens, batch.seq_slot, out.data, rows_of(out, "out"),
+                                batch.n_seqs, static_cast<int>(W), stream), "lru_scan");
+}
+
+// ---------------------------------------------------------------------------- attention with a distance bias
+static void check_kv_wide(const KVView& kv, int kv_heads, int head_dim, int v_dim, DType dtype, const char* who) {
+    need(kv.kv_heads == kv_heads && kv.head_dim == head_dim && kv.v_head_dim == v_dim,
+         std::string(who) + ": the cache has other head sizes than the mixer");
+    need(kv.k && kv.v && kv.table, std::string(who) + ": the cache has no device memory");
+    need(kv.dtype == dtype, std::string(who) + ": the cache holds " + dtype_name(kv.dtype) + ", the rows are " + dtype_name(dtype));
+    need(kv.layer >= 0 && kv.layer < kv.n_layers, std::string(who) + ": layer index outside the cache");
+}
+
+void Ops::kv_store(const Tensor& k, const Tensor& v, const StepBatch& batch, const KVView& kv) {
+    dev(k, "k");
+    dev(v, "v", k.dtype, false);
+    check_kv_wide(kv, kv.kv_heads, kv.head_dim, kv.v_head_dim, k.dtype, "kv_store");
+    const long long T = batch.n_tokens;
+    need(k.ndim == 2 && v.ndim == 2 && k.shape[0] == T && v.shape[0] == T &&
+             k.shape[1] == static_cast<long long>(kv.kv_heads) * kv.head_dim &&
+             v.shape[1] == static_cast<long long>(kv.kv_heads) * kv.v_head_dim,
+         "kv_store: k [rows, kv_heads * head_dim], v [rows, kv_heads * v_dim]");
+    kernel_check(celeg_kv_store(k.data, rows_of(k, "k"), v.data, rows_of(v, "v"), dt(k, "k"), kv.k, kv.v, kv.table, kv.table_stride,
+                                batch.token_slot, batch.positions, static_cast<int>(T), kv.kv_heads, kv.head_dim, kv.v_head_dim,
+                                kv.page_tokens, kv.n_layers, kv.layer, stream), "kv_store");
+}
+
+void Ops::biased_attention(const Tensor& q, const Tensor& out, const ScoreShape& s, const Tensor* r1, const Tensor* r2,
+                           const Tensor* gate, const StepBatch& batch, const KVView& kv, Workspace& ws) {
+    dev(q, "q");
+    dev(out, "out", q.dtype, false);
+    need(s.heads > 0 && s.kv_heads > 0 && s.heads % s.kv_heads == 0 && s.head_dim > 0 && s.v_dim > 0,
+         "biased_attention: heads must be a positive multiple of kv_heads, sizes positive");
+    check_kv_wide(kv, s.kv_heads, s.head_dim, s.v_dim, q.dtype, "biased_attention");
+    const long long T = batch.n_tokens;
+    need(q.ndim == 2 && out.ndim == 2 && q.shape[0] == T && out.shape[0] == T &&
+             q.shape[1] == static_cast<long long>(s.heads) * s.head_dim && out.shape[1] == static_cast<long long>(s.heads) * s.v_dim,
+         "biased_attention: q [rows, heads * head_dim], out [rows, heads * v_dim]");
+    need(s.v_dim <= 256 && s.head_dim <= 1024, "biased_attention: values of up to 256, keys of up to 1,024 numbers a head");
+    need((r1 == nullptr) == (r2 == nullptr), "biased_attention: the distance bias needs both of its numbers per head");
+    if (r1) {
+        dev(*r1, "r1", DType::F32);
+        dev(*r2, "r2", DType::F32);
+        need(r1->numel() == s.heads && r2->numel() == s.heads, "biased_attention: one pair of bias numbers per head");
+    }
+    need(s.every >= 0 && s.window >= 0, "biased_attention: every and window are not negative");
+    if (gate) {
+        dev(*gate, "gate", q.dtype, false);
+        need(gate->ndim == 2 && gate->shape[0] == T && gate->shape[1] == out.shape[1], "biased_attention: gate [rows, heads * v_dim]");
+    }
+    (void)ws;
+    took(Path::AttentionBiased);
+    kernel_check(celeg_biased_attention(q.data, rows_of(q, "q"), dt(q, "q"), kv.k, kv.v, kv.table, kv.table_stride, batch.token_slot,
+                                        batch.positions, r1 ? r1->as<float>() : nullptr, r2 ? r2->as<float>() : nullptr,
+                                        gate ? gate->data : nullptr, gate ? rows_of(*gate, "gate") : 0, out.data, rows_of(out, "out"),
+                                        static_cast<int>(T), s.heads, s.kv_heads, s.head_dim, s.v_dim, kv.page_tokens, kv.n_layers,
+                                        kv.layer, s.scale, s.coef, s.every, s.window, stream), "biased_attention");
+}
+
+// ---------------------------------------------------------------------------- layer glue
+void Ops::activation_bias(const Tensor& x, const Tensor* bias, const Tensor& out, int act) {
+    dev(x, "x");
+    dev(out, "out", x.dtype, false);
+    need(x.ndim == 2 && out.ndim == 2 && x.shape[0] == out.shape[0] && x.shape[1] == out.shape[1], "activation_bias: x and out differ");
+    need(act >= 0 && act <= 2, "activation_bias: act is 0 (gelu), 1 (square of relu) or 2 (none)");
+    if (bias) {
+        dev(*bias, "bias", DType::F32);
+        need(bias->numel() == x.shape[1], "activation_bias: one bias per column");
+    }
+    kernel_check(celeg_activation_bias(x.data, rows_of(x, "x"), bias ? bias->as<float>() : nullptr, out.data, rows_of(out, "out"),
+                                       dt(x, "x"), static_cast<int>(x.shape[0]), static_cast<int>(x.shape[1]), act, stream),
+                 "activation_bias");
+}
+
+void Ops::residual_sum(const Tensor& h, const Tensor& a, const Tensor* b, const Tensor* copy) {
+    dev(h, "h", DType::F32);
+    dev(a, "a");
+    const long long T = h.shape[0], W = h.shape[1];
+    need(h.ndim == 2 && a.ndim == 2 && a.shape[0] == T && a.shape[1] == W, "residual_sum: a must have the stream's shape");
+    if (b) {
+        dev(*b, "b", a.dtype, false);
+        need(b->ndim == 2 && b->shape[0] == T && b->shape[1] == W, "residual_sum: b must have the stream's shape");
+    }
+    if (copy) {
+        dev(*copy, "copy", a.dtype);
+        need(copy->numel() == T * W, "residual_sum: copy must have the stream's shape");
+    }
+    kernel_check(celeg_residual_sum(h.as<float>(), a.data, rows_of(a, "a"), b ? b->data : nullptr, b ? rows_of(*b, "b") : 0,
+                                    copy ? copy->data : nullptr, dt(a, "a"), static_cast<int>(T), static_cast<int>(W), stream),
+                 "residual_sum");
+}
+
+void Ops::token_gate(const Tensor& z, const Tensor& table, int offset, const int* token_ids, const Tensor& g) {
+    dev(z, "z");
+    dev(table, "table", z.dtype);
+    dev(g, "g", z.dtype);
+    need(z.ndim == 2 && table.ndim == 2 && g.ndim == 2 && g.shape[0] == z.shape[0] && g.shape[1] == z.shape[1] && offset >= 0 &&
+             offset + z.shape[1] <= table.shape[1], "token_gate: z and g [rows, dim], the table's rows hold columns [offset, offset + dim)");
+    kernel_check(celeg_token_gate(z.data, rows_of(z, "z"), table.data, rows_of(table, "table"), offset, token_ids, g.data, dt(z, "z"),
+                                  static_cast<int>(z.shape[0]), static_cast<int>(z.shape[1]), stream), "token_gate");
+}
+
+void Ops::normed_mean(const Tensor& a, const Tensor& wa, const Tensor& b, const Tensor& wb, float eps, float factor, const Tensor& out) {
+    dev(a, "a");
+    dev(b, "b", a.dtype, false);
+    dev(out, "out", a.dtype);
+    dev(wa, "wa", DType::F32);
+    dev(wb, "wb", DType::F32);
+    const long long T = a.shape[0], W = a.shape[1];
+    need(a.ndim == 2 && b.ndim == 2 && b.shape[0] == T && b.shape[1] == W && out.numel() == T * W && wa.numel() == W && wb.numel() == W,
+         "normed_mean: a, b and out [rows, width], weights [width]");
+    kernel_check(celeg_normed_mean(a.data, rows_of(a, "a"), wa.as<float>(), b.data, rows_of(b, "b"), wb.as<float>(), eps, factor, out.data,
+                                   dt(a, "a"), static_cast<int>(T), static_cast<int>(W), stream), "normed_mean");
+}
+
+void Ops::depth_mix(const Tensor& history, const Tensor& h, const Tensor& w, int n) {
+    dev(history, "history", DType::F32);
+    dev(h, "h", DType::F32);
+    dev(w, "w", DType::F32);
+    need(history.ndim == 3 && h.ndim == 2 && history.shape[1] == h.shape[0] && history.shape[2] == h.shape[1] && n >= 1 &&
+             n <= history.shape[0] && w.numel() == n, "depth_mix: history [entries >= n, rows, width], w [n]");
+    kernel_check(celeg_depth_mix(history.as<float>(), static_cast<size_t>(history.stride[0]), h.as<float>(), w.as<float>(), n,
+                                 static_cast<int>(h.shape[0]), static_cast<int>(h.shape[1]), stream), "depth_mix");
 }
 
 // Where the context of few requests is cut into parts: how many wavefronts a part's workgroup has

@@ -102,7 +102,7 @@ struct StepPrologue {
 // graph records; a replay counts nothing): what tests and tools ask to see that a size took the
 // path it was meant to take.
 enum class Path : int {
-    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionSigmoid, AttentionSigmoidRows, AttentionSigmoidDecode, DeltaRule, AttentionLatent, AttentionLatentRows, AttentionLatentDecode, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
+    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionSigmoid, AttentionSigmoidRows, AttentionSigmoidDecode, DeltaRule, AttentionLatent, AttentionLatentRows, AttentionLatentDecode, AttentionBiased, AttentionBiasedRows, ChannelScan, LinearRecurrentUnit, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
     FusedSliced, FusedRows, FusedStaged, Tiled, TiledQkv, ArgmaxMerged, Count
 };
 const char* path_name(Path p);
@@ -126,6 +126,7 @@ public:
     bool delta_general = false;          // the delta rule's recurrence always by the kernel for any dim
     bool delta_pairs = true;             // the recurrence in registers takes whole blocks of rows two tokens at a time
     bool use_sigmoid_mfma = true;        // bfloat16 attention with sigmoid weights on the matrix cores
+    bool use_biased_mfma = true;         // bfloat16 attention with a distance bias on the matrix cores
     int sigmoid_rows_form = -1;          // -1: by the step's longest portion; 0 tiles of 16 rows, 1 tiles of 64 rows
     bool use_router_kernel = true;       // the router's product inside the routing kernel
     bool use_moe_mfma = true;            // bfloat16 products of routed experts and per-head matrices on the matrix cores
@@ -202,7 +203,51 @@ public:
     void delta_scan(const Tensor& qk, const Tensor& v, const Tensor& beta_decay, const Tensor& state, const Tensor& out,
                     const DeltaShape& shape, const StepBatch& batch, Workspace& ws);
     // out = o / rms(o) * weight * silu(gate) per head; o [rows, heads * vdim] 32-bit, gate a view with dense rows
-    void delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim);
+    // (act: what the gate passes through, 0 silu, 1 sigmoid)
+    void delta_gated_norm(const Tensor& o, const Tensor& weight, const Tensor& gate, float eps, const Tensor& out, int heads, int vdim,
+                          int act = 0);
+    // Matrix states with a decay per key channel, S [dim, vdim] per value head: S <- diag(decay) S;
+    // u = beta (v - S^T k), or u = v where beta is null; S <- S + k u^T; o = S^T q.
+    // decay = exp(-exp(a_log[head]) softplus(z + dt_bias)); z [rows, heads * dim] with dense rows, decay 32-bit
+    void channel_decay(const Tensor& z, const Tensor& a_log, const Tensor& dt_bias, const Tensor& decay, int heads, int dim);
+    // q, k [rows, heads * dim], v [rows, heads * vdim] and z [rows, heads * dim] (views with dense rows) -> qk (q times
+    // q_scale | k), v32 and decay = sigmoid(z + z_bias)^(1 / tau), all 32-bit
+    void gla_prepare(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& z, const Tensor* z_bias, float tau, float q_scale,
+                     const Tensor& qk, const Tensor& v32, const Tensor& decay);
+    // qk [rows, 2 * kv_heads * dim], v and out [rows, heads * vdim], decay [rows, heads * dim]; beta: entry
+    // [row * beta_ld + head] of a 32-bit buffer, or null; state [slots, heads, dim, vdim] (shape.taps is not read)
+    void channel_scan(const Tensor& qk, const Tensor& v, const Tensor& decay, const float* beta, int beta_ld, const Tensor& state,
+                      const Tensor& out, const DeltaShape& shape, const StepBatch& batch);
+    // The real-gated linear recurrent unit over `width` channels in `blocks` equal parts, a causal
+    // convolution of `taps` in front.  x: the convolution's inputs [rows, width] (a view with dense rows);
+    // ra_t, ri_t [blocks, in, out] 32-bit; leaves decay a and input sqrt(1 - a^2) i u [rows, width] 32-bit and
+    // moves the requests' saved inputs [slots, taps - 1, width] on.
+    struct LruShape { int width = 0, blocks = 0, taps = 0; float decay_scale = 8.f; };   // log a = -decay_scale r softplus(lam)
+    void lru_gates(const Tensor& x, const Tensor& conv_w, const Tensor* conv_b, const Tensor& ra_t, const Tensor& ra_b,
+                   const Tensor& ri_t, const Tensor& ri_b, const Tensor& lam, const Tensor& conv_state, const Tensor& decay,
+                   const Tensor& input, const LruShape& shape, const StepBatch& batch);
+    // S <- a S + input per channel from and into state [slots, width]; out = S * gelu_tanh(y)
+    void lru_scan(const Tensor& decay, const Tensor& input, const Tensor& y, const Tensor& state, const Tensor& out,
+                  const StepBatch& batch);
+    // Softmax attention whose positions enter through the scores: score = (q . k) * scale * f(i) - r1[h] ln(1 + r2[h] (i - j)),
+    // f(i) = 1 + coef ln(floor((i + 1) / every) + 1) (every 0: f = 1); r1, r2 [heads] 32-bit or null.  Values of kv.v_head_dim.
+    // gate: raw values [rows, heads * v_dim] (a view with dense rows) whose sigmoid multiplies the result, or null.
+    struct ScoreShape { int heads = 0, kv_heads = 0, head_dim = 0, v_dim = 0, window = 0, every = 0; float scale = 1.f, coef = 0.f; };
+    // a step's keys [rows, kv_heads * head_dim] and values [rows, kv_heads * v_dim] to their places in the pages
+    void kv_store(const Tensor& k, const Tensor& v, const StepBatch& batch, const KVView& kv);
+    void biased_attention(const Tensor& q, const Tensor& out, const ScoreShape& shape, const Tensor* r1, const Tensor* r2,
+                          const Tensor* gate, const StepBatch& batch, const KVView& kv, Workspace& ws);
+    // layer glue (32-bit arithmetic; rows of the run's dtype)
+    // out = act(x + bias): act 0 gelu (tanh form), 1 square of relu, 2 none; x and out views with dense rows
+    void activation_bias(const Tensor& x, const Tensor* bias, const Tensor& out, int act);
+    // h += a (+ b), h the 32-bit stream; copy (or null) receives the new rows in the run's dtype
+    void residual_sum(const Tensor& h, const Tensor& a, const Tensor* b, const Tensor* copy);
+    // g[t, j] = gelu_tanh(z[t, j]) * table[token[t], offset + j]
+    void token_gate(const Tensor& z, const Tensor& table, int offset, const int* token_ids, const Tensor& g);
+    // out = factor * (rmsnorm(a) * wa + rmsnorm(b) * wb) row by row
+    void normed_mean(const Tensor& a, const Tensor& wa, const Tensor& b, const Tensor& wb, float eps, float factor, const Tensor& out);
+    // history [entries, rows, width] 32-bit: entry n - 1 becomes the stream h, and h becomes sum_{j < n} w[j] history[j]
+    void depth_mix(const Tensor& history, const Tensor& h, const Tensor& w, int n);
     // whether a decode-only step's attention can prepare and write the step's own keys and values itself
     bool attention_fresh_ok(int heads, int head_dim, const Tensor* inv_freq, int rotary_dim, int pairing, const StepBatch& batch,
                             const KVView& kv, DType dtype) const;
@@ -243,7 +288,8 @@ public:
     }
     void moe_gather(const Tensor& x, const RoutePlan& plan, bool weighted, const Tensor& a);
     // out[p] = a[p] w[expert of p]^T; w [experts * N, K], or [experts * 2N, K] if gated (silu(gate) * up)
-    void moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool gated, const RoutePlan& plan);
+    // (not gated, act 1: the square of relu of the product)
+    void moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool gated, const RoutePlan& plan, int act = 0);
     void moe_combine(const Tensor& y, const RoutePlan& plan, bool weighted, const Tensor& out);
     // sampling
     void sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen,
@@ -314,6 +360,8 @@ struct Runtime {
     // the stream's bfloat16 copy is; whoever writes the stream another way resets them
     int stream_stat_blocks = 0;
     bool stream_has_bf16 = false;
+    // the stream's rows in the run's dtype, where whoever wrote the stream last left them (undefined: nobody did)
+    Tensor stream_copy;
     // the step's prologue, left by the runner for the embedding's kernel to take along
     // (defer_prologue); whoever cannot take it along calls flush_prologue() before its own work
     bool defer_prologue = true;

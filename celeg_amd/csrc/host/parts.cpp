@@ -713,7 +713,8 @@ private:
 // matrix is held in 32-bit); "score": "sigmoid" (s = 1 / (1 + e^-z), every expert by itself) or
 // "softmax" (over all experts); the `top` largest are chosen, their scores are the weights
 // ("renormalize": divided by their sum).  "weight_on": "input" (the output is
-// sum expert(w x)) or "output" (sum w expert(x)).
+// sum expert(w x)) or "output" (sum w expert(x)).  "gated": false makes an expert
+// W_down act(W_up x) with "activation": "relu2" (the square of relu) and no gate matrix.
 class RoutedExperts final : public FeedForward {
 public:
     explicit RoutedExperts(const PartSpec& s) : FeedForward(s) {
@@ -728,6 +729,10 @@ public:
         score_ = score == "softmax" ? 1 : 0;
         on_input_ = on == "input";
         renorm_ = p.get_bool("renormalize", false);
+        gated_ = p.get_bool("gated", true);
+        const std::string act = p.get_string("activation", gated_ ? "silu" : "relu2");
+        if (act != (gated_ ? "silu" : "relu2"))
+            throw SpecError("routed_experts: activation is 'silu' for gated experts and 'relu2' for experts without a gate, not '" + act + "'");
         if (width_ <= 0 || ff_ <= 0 || experts_ <= 0 || top_ <= 0 || top_ > experts_)
             throw SpecError("routed_experts: width, ff and experts must be positive and top between 1 and experts");
     }
@@ -736,7 +741,7 @@ public:
     WeightSpecs weight_specs() const override {
         WeightSpecs specs{{"router", WeightSpec{{experts_, width_}, "vector", "normal", {}}}};
         for (int e = 0; e < experts_; ++e) {
-            specs.push_back({role("gate", e), matrix(ff_, width_)});
+            if (gated_) specs.push_back({role("gate", e), matrix(ff_, width_)});
             specs.push_back({role("up", e), matrix(ff_, width_)});
             specs.push_back({role("down", e), matrix(width_, ff_)});
         }
@@ -746,13 +751,13 @@ public:
         router_ = get(t, "router");
         std::vector<std::shared_ptr<DeviceTensor>> in, out;
         for (int e = 0; e < experts_; ++e) {
-            in.push_back(get(t, role("gate", e)));
+            if (gated_) in.push_back(get(t, role("gate", e)));
             in.push_back(get(t, role("up", e)));
             out.push_back(get(t, role("down", e)));
         }
         for (const auto& w : in)
             if (w->view.dtype != in[0]->view.dtype) throw SpecError("routed_experts: the experts are stored in different dtypes");
-        w_gate_up_ = concat_rows(in);       // [experts * 2 ff, width]: per expert its gate rows, then its up rows
+        w_gate_up_ = concat_rows(in);       // [experts * 2 ff, width]: per expert its gate rows, then its up rows (no gate: [experts * ff, width])
         w_down_ = concat_rows(out);         // [experts * width, ff]
     }
     Tensor forward(const Tensor& x, const StepBatch&, Runtime& rt) override {
@@ -763,7 +768,7 @@ public:
         Tensor a = rt.ws.buf("moe_in", rt.dtype, {T * top_, width_});
         rt.ops.moe_gather(x, plan, on_input_, a);
         Tensor act = rt.ws.buf("moe_act", rt.dtype, {T * top_, ff_});
-        rt.ops.moe_product(a, w_gate_up_->view, act, true, plan);
+        rt.ops.moe_product(a, w_gate_up_->view, act, gated_, plan, gated_ ? 0 : 1);
         Tensor y = rt.ws.buf("moe_y", rt.dtype, {T * top_, width_});
         rt.ops.moe_product(act, w_down_->view, y, false, plan);
         Tensor out = rt.ws.buf("ffn_out", rt.dtype, {T, width_});
@@ -774,7 +779,7 @@ public:
 private:
     long long width_ = 0, ff_ = 0;
     int experts_ = 0, top_ = 0, score_ = 0;
-    bool on_input_ = false, renorm_ = false;
+    bool on_input_ = false, renorm_ = false, gated_ = true;
     std::shared_ptr<DeviceTensor> router_, w_gate_up_, w_down_;
 };
 
@@ -1249,6 +1254,39 @@ private:
     std::shared_ptr<DeviceTensor> w_in_, b_in_, w_o_, q_norm_, k_norm_, temp_, pb_;
 };
 
+// ---------------------------------------------------------------------------- projections side by side
+// The matrices of several projections of one input, one under the other, so that one product
+// makes them all.  A piece that a later product reads as its input starts at a multiple of 16
+// rows (zero rows in front of it); the whole is padded to a multiple of 16 rows.
+struct Stacked {
+    std::shared_ptr<DeviceTensor> weight;
+    std::vector<long long> at;        // the first row of every piece
+    long long rows = 0;
+};
+Stacked stack_projections(const std::vector<std::pair<std::shared_ptr<DeviceTensor>, bool>>& pieces, const char* who) {
+    Stacked out;
+    std::vector<std::shared_ptr<DeviceTensor>> parts;
+    const DType dtype = pieces.at(0).first->view.dtype;
+    const long long width = pieces.at(0).first->view.shape[1];
+    auto pad_to_16 = [&]() {
+        const long long pad = (16 - out.rows % 16) % 16;
+        if (pad) parts.push_back(from_host_floats(std::vector<float>(static_cast<size_t>(pad * width), 0.f), dtype, {pad, width}));
+        out.rows += pad;
+    };
+    for (const auto& piece : pieces) {
+        const Tensor& v = piece.first->view;
+        if (v.dtype != dtype || v.ndim != 2 || v.shape[1] != width)
+            throw SpecError(std::string(who) + ": the input projections differ in dtype or inner size");
+        if (piece.second) pad_to_16();
+        out.at.push_back(out.rows);
+        parts.push_back(piece.first);
+        out.rows += v.shape[0];
+    }
+    pad_to_16();
+    out.weight = concat_rows(parts);
+    return out;
+}
+
 // ---------------------------------------------------------------------------- gated delta rule
 // A recurrent mixer with a matrix of state per head.
 //
@@ -1256,11 +1294,15 @@ private:
 // query/key head i / (heads / kv_heads)); each channel of q, k and v passes a short causal
 // convolution over time (taps [channels, taps], the last tap the current token's, zeros before
 // the sequence starts) and silu; q and k become unit vectors per head
-// (x / sqrt(sum x^2 + 1e-6)), q times dim^-1/2.  beta = sigmoid(W_b h) and the decay
-// a = exp(-exp(A_log) softplus(W_a h + dt_bias)), one each per value head.  Per head and token
-//     S <- a S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// (x / sqrt(sum x^2 + 1e-6)), q times dim^-1/2.  beta = sigmoid(W_b h), one per value head.
+// The decay is exp(-exp(A_log[head]) softplus(z + dt_bias)) with "decay": "head" (one per value
+// head, z = W_a h, dt_bias [heads]) or "channel" (one per value head and key channel, acting on
+// the rows of S; z and dt_bias [heads * dim]).  "decay_rank" r > 0: z = W_a2 (W_a1 h) through r
+// values (tensors a1, a2 instead of a).  Per head and token
+//     S <- decay S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 // so the read-out sees the token's own write.  o is RMS-normed per head over vdim (weight
-// [vdim] shared by the heads) and multiplied by silu(W_g h); the heads go through W_o.
+// [vdim] shared by the heads) and multiplied by act(W_g h), "gate": "silu" or "sigmoid";
+// "gate_rank" r > 0: W_g2 (W_g1 h) (tensors g1, g2 instead of g).  The heads go through W_o.
 //
 // State per request: S [heads, dim, vdim] and the last taps - 1 inputs of the convolutions
 // [taps - 1, channels], both 32-bit.  Everything from the convolutions' sums to the gated norm
@@ -1276,42 +1318,64 @@ public:
         shape_.vdim = static_cast<int>(p.get_int("vdim", shape_.dim));
         shape_.taps = static_cast<int>(p.get_int("taps", 0));
         eps_ = static_cast<float>(p.get_double("eps", 1e-6));
+        const std::string decay = p.get_string("decay", "head"), gate = p.get_string("gate", "silu");
+        if (decay != "head" && decay != "channel") throw SpecError("gated_delta_rule: decay is 'head' or 'channel', not '" + decay + "'");
+        if (gate != "silu" && gate != "sigmoid") throw SpecError("gated_delta_rule: gate is 'silu' or 'sigmoid', not '" + gate + "'");
+        per_channel_ = decay == "channel";
+        gate_act_ = gate == "sigmoid" ? 1 : 0;
+        decay_rank_ = p.get_int("decay_rank", 0);
+        gate_rank_ = p.get_int("gate_rank", 0);
         if (width_ <= 0 || shape_.heads <= 0 || shape_.kv_heads <= 0 || shape_.heads % shape_.kv_heads)
             throw SpecError("gated_delta_rule: heads must be a positive multiple of kv_heads");
         if (shape_.dim <= 0 || shape_.vdim <= 0 || shape_.taps <= 0) throw SpecError("gated_delta_rule: dim, vdim and taps must be positive");
+        if (decay_rank_ < 0 || gate_rank_ < 0) throw SpecError("gated_delta_rule: decay_rank and gate_rank are not negative");
+        if (decay_rank_ > 0 && !per_channel_) throw SpecError("gated_delta_rule: decay_rank goes with decay 'channel'");
     }
     bool graph_safe() const override { return true; }
     long long qk_width() const { return static_cast<long long>(shape_.kv_heads) * shape_.dim; }
     long long v_width() const { return static_cast<long long>(shape_.heads) * shape_.vdim; }
     long long channels() const { return 2 * qk_width() + v_width(); }
+    long long decay_width() const { return per_channel_ ? static_cast<long long>(shape_.heads) * shape_.dim : shape_.heads; }
     std::vector<StateNeed> state_needs() const override {
         return {StateNeed{"S", {shape_.heads, shape_.dim, shape_.vdim}, DType::F32},
                 StateNeed{"conv", {std::max(shape_.taps - 1, 1), channels()}, DType::F32}};
     }
     WeightSpecs weight_specs() const override {
         auto taps = [&](long long n) { return WeightSpec{{n, shape_.taps}, "vector", "normal", {}}; };
-        return {{"q", matrix(qk_width(), width_)}, {"k", matrix(qk_width(), width_)}, {"v", matrix(v_width(), width_)},
-                {"q_conv", taps(qk_width())},      {"k_conv", taps(qk_width())},      {"v_conv", taps(v_width())},
-                {"b", matrix(shape_.heads, width_)}, {"a", matrix(shape_.heads, width_)}, {"A_log", vec(shape_.heads)},
-                {"dt_bias", vec(shape_.heads)},    {"norm", vec(shape_.vdim, "around_one")}, {"g", matrix(v_width(), width_)},
-                {"o", matrix(width_, v_width())}};
+        WeightSpecs specs{{"q", matrix(qk_width(), width_)}, {"k", matrix(qk_width(), width_)}, {"v", matrix(v_width(), width_)},
+                          {"q_conv", taps(qk_width())},      {"k_conv", taps(qk_width())},      {"v_conv", taps(v_width())},
+                          {"b", matrix(shape_.heads, width_)}, {"A_log", vec(shape_.heads)},    {"dt_bias", vec(decay_width())},
+                          {"norm", vec(shape_.vdim, "around_one")}, {"o", matrix(width_, v_width())}};
+        if (decay_rank_ > 0) {
+            specs.push_back({"a1", matrix(decay_rank_, width_)});
+            specs.push_back({"a2", matrix(decay_width(), decay_rank_)});
+        } else {
+            specs.push_back({"a", matrix(decay_width(), width_)});
+        }
+        if (gate_rank_ > 0) {
+            specs.push_back({"g1", matrix(gate_rank_, width_)});
+            specs.push_back({"g2", matrix(v_width(), gate_rank_)});
+        } else {
+            specs.push_back({"g", matrix(v_width(), width_)});
+        }
+        return specs;
     }
     void load(const PartTensors& t, Runtime&) override {
         // one product for everything that reads the mixer's input: q | k | v | gate | b | a (| zero rows)
-        std::vector<std::shared_ptr<DeviceTensor>> in{get(t, "q"), get(t, "k"), get(t, "v"), get(t, "g"), get(t, "b"), get(t, "a")};
-        for (const auto& w : in)
-            if (w->view.dtype != in[0]->view.dtype) throw SpecError("gated_delta_rule: the input projections are stored in different dtypes");
-        col_gate_ = channels();
-        col_b_ = col_gate_ + v_width();
-        col_a_ = col_b_ + shape_.heads;
-        const long long cols = col_a_ + shape_.heads, pad = (16 - cols % 16) % 16;
-        if (pad) in.push_back(from_host_floats(std::vector<float>(static_cast<size_t>(pad * width_), 0.f), in[0]->view.dtype, {pad, width_}));
-        w_in_ = concat_rows(in);
+        const Stacked in = stack_projections({{get(t, "q"), false}, {get(t, "k"), false}, {get(t, "v"), false},
+                                              {get(t, gate_rank_ > 0 ? "g1" : "g"), gate_rank_ > 0}, {get(t, "b"), false},
+                                              {get(t, decay_rank_ > 0 ? "a1" : "a"), decay_rank_ > 0}}, "gated_delta_rule");
+        w_in_ = in.weight;
+        col_gate_ = in.at[3];
+        col_b_ = in.at[4];
+        col_a_ = in.at[5];
         conv_w_ = concat_rows({get(t, "q_conv"), get(t, "k_conv"), get(t, "v_conv")});
         a_log_ = get(t, "A_log");
         dt_bias_ = get(t, "dt_bias");
         norm_ = get(t, "norm");
         w_o_ = get(t, "o");
+        a2_ = maybe(t, "a2");
+        g2_ = maybe(t, "g2");
     }
     Tensor forward(const Tensor& x, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
         const long long T = x.shape[0];
@@ -1320,22 +1384,42 @@ public:
         Tensor qk = rt.ws.buf("delta_qk", DType::F32, {T, 2 * qk_width()});
         Tensor v = rt.ws.buf("delta_v", DType::F32, {T, v_width()});
         Tensor beta_decay = rt.ws.buf("delta_beta_decay", DType::F32, {T, 2LL * shape_.heads});
-        rt.ops.delta_prepare(proj, static_cast<int>(col_b_), static_cast<int>(col_a_), shape_, conv_w_->view, a_log_->view,
-                             dt_bias_->view, cache.states.at("conv"), qk, v, beta_decay, batch);
         Tensor o = rt.ws.buf("delta_o", DType::F32, {T, v_width()});
-        rt.ops.delta_scan(qk, v, beta_decay, cache.states.at("S"), o, shape_, batch, rt.ws);
+        if (!per_channel_) {
+            rt.ops.delta_prepare(proj, static_cast<int>(col_b_), static_cast<int>(col_a_), shape_, conv_w_->view, a_log_->view,
+                                 dt_bias_->view, cache.states.at("conv"), qk, v, beta_decay, batch);
+            rt.ops.delta_scan(qk, v, beta_decay, cache.states.at("S"), o, shape_, batch, rt.ws);
+        } else {
+            Tensor z = proj.cols(col_a_, decay_width());
+            if (decay_rank_ > 0) {
+                z = rt.ws.buf("delta_decay_in", rt.dtype, {T, decay_width()});
+                rt.ops.linear(proj.cols(col_a_, decay_rank_), a2_->view, z, nullptr, rt.ws);
+            }
+            Tensor decay = rt.ws.buf("delta_decay", DType::F32, {T, decay_width()});
+            rt.ops.channel_decay(z, a_log_->view, dt_bias_->view, decay, shape_.heads, shape_.dim);
+            rt.ops.delta_prepare(proj, static_cast<int>(col_b_), static_cast<int>(col_b_), shape_, conv_w_->view, Tensor(), Tensor(),
+                                 cache.states.at("conv"), qk, v, beta_decay, batch);
+            rt.ops.channel_scan(qk, v, decay, beta_decay.as<float>(), 2 * shape_.heads, cache.states.at("S"), o, shape_, batch);
+        }
+        Tensor gate = proj.cols(col_gate_, v_width());
+        if (gate_rank_ > 0) {
+            gate = rt.ws.buf("delta_gate", rt.dtype, {T, v_width()});
+            rt.ops.linear(proj.cols(col_gate_, gate_rank_), g2_->view, gate, nullptr, rt.ws);
+        }
         Tensor gated = rt.ws.buf("delta_gated", rt.dtype, {T, v_width()});
-        rt.ops.delta_gated_norm(o, norm_->view, proj.cols(col_gate_, v_width()), eps_, gated, shape_.heads, shape_.vdim);
+        rt.ops.delta_gated_norm(o, norm_->view, gate, eps_, gated, shape_.heads, shape_.vdim, gate_act_);
         Tensor out = rt.ws.buf("mixer_out", rt.dtype, {T, width_});
         rt.ops.linear(gated, w_o_->view, out, nullptr, rt.ws);
         return out;
     }
 
 private:
-    long long width_ = 0, col_gate_ = 0, col_b_ = 0, col_a_ = 0;
+    long long width_ = 0, col_gate_ = 0, col_b_ = 0, col_a_ = 0, decay_rank_ = 0, gate_rank_ = 0;
     Ops::DeltaShape shape_;
     float eps_ = 1e-6f;
-    std::shared_ptr<DeviceTensor> w_in_, conv_w_, a_log_, dt_bias_, norm_, w_o_;
+    bool per_channel_ = false;
+    int gate_act_ = 0;
+    std::shared_ptr<DeviceTensor> w_in_, conv_w_, a_log_, dt_bias_, norm_, w_o_, a2_, g2_;
 };
 
 // ---------------------------------------------------------------------------- the embedding's rows, again
@@ -1420,6 +1504,487 @@ private:
     std::unique_ptr<Norm> ffn_post_;
 };
 
+// ---------------------------------------------------------------------------- attention with a distance bias
+// Grouped-query softmax attention without a rotation: positions enter through the scores alone.
+//
+// q = W_q h, k = W_k h (head_dim a head), v = W_v h ("v_dim" a head, which may differ from head_dim).
+// score(i, j) = (q_i . k_j) * scale * f(i) - r1[h] ln(1 + r2[h] (i - j)) with
+// f(i) = 1 + coef ln(floor((i + 1) / every) + 1) ("query_temperature": {"coef", "every"}; absent: f = 1) and,
+// with "distance_bias", a learned pair (r1, r2) per query head.  Keys j <= i (inside "window" where one is
+// given).  "gate": "sigmoid" multiplies the heads, side by side, element by element with sigmoid(W_g h).
+class BiasedAttention final : public Mixer {
+public:
+    explicit BiasedAttention(const PartSpec& s) : Mixer(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        shape_.heads = static_cast<int>(p.get_int("heads", 0));
+        shape_.kv_heads = static_cast<int>(p.get_int("kv_heads", shape_.heads));
+        shape_.head_dim = static_cast<int>(p.get_int("head_dim", 0));
+        shape_.v_dim = static_cast<int>(p.get_int("v_dim", shape_.head_dim));
+        if (width_ <= 0 || shape_.heads <= 0 || shape_.kv_heads <= 0 || shape_.heads % shape_.kv_heads)
+            throw SpecError("biased_attention: heads must be a positive multiple of kv_heads");
+        if (shape_.head_dim <= 0 || shape_.v_dim <= 0) throw SpecError("biased_attention: head_dim and v_dim must be positive");
+        shape_.scale = p["scale"].is_null() ? static_cast<float>(1.0 / std::sqrt(static_cast<double>(shape_.head_dim)))
+                                            : static_cast<float>(p["scale"].as_double());
+        if (!p["window"].is_null()) {
+            shape_.window = static_cast<int>(p["window"].as_int());
+            if (shape_.window <= 0) throw SpecError("biased_attention: window must be positive");
+        }
+        if (!p["query_temperature"].is_null()) {
+            const Json& t = p["query_temperature"];
+            shape_.coef = static_cast<float>(t.get_double("coef", 0.0));
+            shape_.every = static_cast<int>(t.get_int("every", 0));
+            if (shape_.every <= 0) throw SpecError("biased_attention: query_temperature.every must be positive");
+        }
+        distance_bias_ = p.get_bool("distance_bias", false);
+        const std::string gate = p.get_string("gate", "none");
+        if (gate != "none" && gate != "sigmoid") throw SpecError("biased_attention: gate is 'none' or 'sigmoid', not '" + gate + "'");
+        gated_ = gate == "sigmoid";
+    }
+    bool graph_safe() const override { return true; }
+    std::optional<KVNeed> kv_need() const override {
+        KVNeed need{shape_.kv_heads, shape_.head_dim, shape_.window > 0 ? std::optional<int>(shape_.window) : std::nullopt};
+        need.v_head_dim = shape_.v_dim;
+        return need;
+    }
+    long long q_width() const { return static_cast<long long>(shape_.heads) * shape_.head_dim; }
+    long long k_width() const { return static_cast<long long>(shape_.kv_heads) * shape_.head_dim; }
+    long long v_width() const { return static_cast<long long>(shape_.kv_heads) * shape_.v_dim; }
+    long long o_width() const { return static_cast<long long>(shape_.heads) * shape_.v_dim; }
+    WeightSpecs weight_specs() const override {
+        WeightSpecs specs{{"q", matrix(q_width(), width_)}, {"k", matrix(k_width(), width_)}, {"v", matrix(v_width(), width_)},
+                          {"o", matrix(width_, o_width())}};
+        if (distance_bias_) {
+            specs.push_back({"r1", vec(shape_.heads)});
+            specs.push_back({"r2", vec(shape_.heads, "around_one")});
+        }
+        if (gated_) specs.push_back({"g", matrix(o_width(), width_)});
+        return specs;
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        std::vector<std::pair<std::shared_ptr<DeviceTensor>, bool>> pieces{{get(t, "q"), false}, {get(t, "k"), false}, {get(t, "v"), false}};
+        if (gated_) pieces.push_back({get(t, "g"), false});
+        const Stacked in = stack_projections(pieces, "biased_attention");
+        w_in_ = in.weight;
+        col_k_ = in.at[1];
+        col_v_ = in.at[2];
+        col_g_ = gated_ ? in.at[3] : 0;
+        w_o_ = get(t, "o");
+        r1_ = maybe(t, "r1");
+        r2_ = maybe(t, "r2");
+    }
+    Tensor forward(const Tensor& x, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        if (!cache.kv) throw SpecError("biased_attention: the cache has no keys and values for this layer");
+        if (!cache.writes_kv) throw SpecError("biased_attention: reading another entry's cache is not supported");
+        const long long T = x.shape[0];
+        Tensor proj = rt.ws.buf("battn_proj", rt.dtype, {T, w_in_->view.shape[0]});
+        rt.ops.linear(x, w_in_->view, proj, nullptr, rt.ws);
+        // every row's keys and values are in their pages before any row attends
+        rt.ops.kv_store(proj.cols(col_k_, k_width()), proj.cols(col_v_, v_width()), batch, *cache.kv);
+        Tensor attended = rt.ws.buf("battn_out", rt.dtype, {T, o_width()});
+        Tensor gate = gated_ ? proj.cols(col_g_, o_width()) : Tensor();
+        rt.ops.biased_attention(proj.cols(0, q_width()), attended, shape_, r1_ ? &r1_->view : nullptr, r2_ ? &r2_->view : nullptr,
+                                gated_ ? &gate : nullptr, batch, *cache.kv, rt.ws);
+        Tensor out = rt.ws.buf("battn_mixer_out", rt.dtype, {T, width_});
+        rt.ops.linear(attended, w_o_->view, out, nullptr, rt.ws);
+        return out;
+    }
+
+private:
+    long long width_ = 0, col_k_ = 0, col_v_ = 0, col_g_ = 0;
+    Ops::ScoreShape shape_;
+    bool distance_bias_ = false, gated_ = false;
+    std::shared_ptr<DeviceTensor> w_in_, w_o_, r1_, r2_;
+};
+
+// ---------------------------------------------------------------------------- real-gated linear recurrent unit
+// A recurrent block with two branches of "inner" channels from the mixer's input h:
+//     y = gelu_tanh(W_y h + b_y);   u = conv(W_x h + b_x)     (a causal convolution per channel with "taps" taps
+//                                                               and a bias, the last tap the current token's)
+// u in "blocks" equal parts; in part b  r = sigmoid(Ra[b] u_b + ra_b), i = sigmoid(Ri[b] u_b + ri_b), square
+// matrices stored [out, in].  log a = -c r softplus(lam) ("decay_scale" c, 8 unless given), a = exp(log a),
+//     S <- a S + sqrt(1 - a^2) (i u)       from S = 0, the first token like every other
+// and the output is W_o (S * y).  State per request: S [inner] and the last taps - 1 inputs of the
+// convolution, both 32-bit; gates, decays and the recurrence are 32-bit.
+class LinearRecurrentUnit final : public Mixer {
+public:
+    explicit LinearRecurrentUnit(const PartSpec& s) : Mixer(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        shape_.width = static_cast<int>(p.get_int("inner", 0));
+        shape_.blocks = static_cast<int>(p.get_int("blocks", 1));
+        shape_.taps = static_cast<int>(p.get_int("taps", 0));
+        shape_.decay_scale = static_cast<float>(p.get_double("decay_scale", 8.0));
+        if (width_ <= 0 || shape_.width <= 0 || shape_.blocks <= 0 || shape_.width % shape_.blocks)
+            throw SpecError("linear_recurrent_unit: inner must be a positive multiple of blocks");
+        if (shape_.taps <= 0) throw SpecError("linear_recurrent_unit: taps must be positive");
+    }
+    bool graph_safe() const override { return true; }
+    std::vector<StateNeed> state_needs() const override {
+        return {StateNeed{"S", {shape_.width}, DType::F32}, StateNeed{"conv", {std::max(shape_.taps - 1, 1), shape_.width}, DType::F32}};
+    }
+    WeightSpecs weight_specs() const override {
+        const long long I = shape_.width, bw = I / shape_.blocks;
+        auto cube = [&]() { return WeightSpec{{shape_.blocks, bw, bw}, "vector", "normal", {}}; };
+        auto per_block = [&]() { return WeightSpec{{shape_.blocks, bw}, "vector", "normal", {}}; };
+        return {{"y", matrix(I, width_)},      {"y_bias", vec(I)},          {"x", matrix(I, width_)},  {"x_bias", vec(I)},
+                {"conv", WeightSpec{{I, shape_.taps}, "vector", "normal", {}}}, {"conv_bias", vec(I)}, {"ra", cube()},
+                {"ra_bias", per_block()},      {"ri", cube()},              {"ri_bias", per_block()},  {"lam", vec(I)},
+                {"o", matrix(width_, I)}};
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        const Stacked in = stack_projections({{get(t, "y"), false}, {get(t, "x"), false}}, "linear_recurrent_unit");
+        w_in_ = in.weight;
+        col_x_ = in.at[1];
+        std::vector<float> b = to_host_floats(get(t, "y_bias")->view), bx = to_host_floats(get(t, "x_bias")->view);
+        b.resize(static_cast<size_t>(col_x_), 0.f);
+        b.insert(b.end(), bx.begin(), bx.end());
+        b.resize(static_cast<size_t>(in.rows), 0.f);
+        b_in_ = from_host_floats(b, DType::F32, {in.rows});
+        conv_w_ = get(t, "conv");
+        conv_b_ = get(t, "conv_bias");
+        // the gate matrices turned over, [blocks, in, out]: neighbouring threads read neighbouring weights
+        const long long bw = shape_.width / shape_.blocks;
+        auto turned = [&](const char* role) {
+            const std::vector<float> w = to_host_floats(get(t, role)->view);
+            std::vector<float> out(w.size());
+            for (long long b2 = 0; b2 < shape_.blocks; ++b2)
+                for (long long o = 0; o < bw; ++o)
+                    for (long long i = 0; i < bw; ++i)
+                        out[static_cast<size_t>((b2 * bw + i) * bw + o)] = w[static_cast<size_t>((b2 * bw + o) * bw + i)];
+            return from_host_floats(out, DType::F32, {shape_.blocks, bw, bw});
+        };
+        ra_t_ = turned("ra");
+        ri_t_ = turned("ri");
+        ra_b_ = get(t, "ra_bias");
+        ri_b_ = get(t, "ri_bias");
+        lam_ = get(t, "lam");
+        w_o_ = get(t, "o");
+    }
+    Tensor forward(const Tensor& x, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        const long long T = x.shape[0], I = shape_.width;
+        Tensor proj = rt.ws.buf("lru_proj", rt.dtype, {T, w_in_->view.shape[0]});
+        rt.ops.linear(x, w_in_->view, proj, &b_in_->view, rt.ws);
+        Tensor decay = rt.ws.buf("lru_decay", DType::F32, {T, I}), input = rt.ws.buf("lru_input", DType::F32, {T, I});
+        rt.ops.lru_gates(proj.cols(col_x_, I), conv_w_->view, &conv_b_->view, ra_t_->view, ra_b_->view, ri_t_->view, ri_b_->view,
+                         lam_->view, cache.states.at("conv"), decay, input, shape_, batch);
+        Tensor gated = rt.ws.buf("lru_gated", rt.dtype, {T, I});
+        rt.ops.lru_scan(decay, input, proj.cols(0, I), cache.states.at("S"), gated, batch);
+        Tensor out = rt.ws.buf("lru_mixer_out", rt.dtype, {T, width_});
+        rt.ops.linear(gated, w_o_->view, out, nullptr, rt.ws);
+        return out;
+    }
+
+private:
+    long long width_ = 0, col_x_ = 0;
+    Ops::LruShape shape_;
+    std::shared_ptr<DeviceTensor> w_in_, b_in_, conv_w_, conv_b_, ra_t_, ri_t_, ra_b_, ri_b_, lam_, w_o_;
+};
+
+// ---------------------------------------------------------------------------- two mixers side by side
+// normed_pair: both mixers ("left" and "right", parts of their own) read the same rows; the result is
+// factor * (rmsnorm(left(h)) * w_left + rmsnorm(right(h)) * w_right) with plain weights over the model
+// width ("factor" 0.5 unless given: the mean).  A child's tensors are this part's, the role prefixed
+// "left." or "right."; so are its states.  At most one of the two keeps keys and values in pages.
+class NormedPair final : public Mixer {
+public:
+    explicit NormedPair(const PartSpec& s) : Mixer(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        eps_ = static_cast<float>(p.get_double("eps", 1e-6));
+        factor_ = static_cast<float>(p.get_double("factor", 0.5));
+        if (width_ <= 0) throw SpecError("normed_pair: width must be positive");
+        const char* sides[2] = {"left", "right"};
+        for (int i = 0; i < 2; ++i) {
+            if (!PartSpec::is_part(p[sides[i]])) throw SpecError(std::string("normed_pair: '") + sides[i] + "' must be a mixer");
+            PartSpec child = PartSpec::from_json(p[sides[i]], std::string("normed_pair.") + sides[i]);
+            const std::string prefix = std::string(sides[i]) + ".";
+            for (const auto& t : s.tensors)
+                if (t.first.rfind(prefix, 0) == 0) child.tensors.emplace_back(t.first.substr(prefix.size()), t.second);
+            child_[i] = build_as<Mixer>("mixer", child);
+        }
+        if (child_[0]->kv_need() && child_[1]->kv_need()) throw SpecError("normed_pair: only one of the two mixers may keep keys and values");
+    }
+    bool graph_safe() const override { return true; }
+    std::vector<const Part*> children() const override { return {child_[0].get(), child_[1].get()}; }
+    std::optional<KVNeed> kv_need() const override { return child_[0]->kv_need() ? child_[0]->kv_need() : child_[1]->kv_need(); }
+    std::vector<StateNeed> state_needs() const override {
+        std::vector<StateNeed> out;
+        for (int i = 0; i < 2; ++i)
+            for (StateNeed n : child_[i]->state_needs()) {
+                n.name = prefix(i) + n.name;
+                out.push_back(std::move(n));
+            }
+        return out;
+    }
+    WeightSpecs weight_specs() const override {
+        WeightSpecs specs{{"left_out", vec(width_, "around_one")}, {"right_out", vec(width_, "around_one")}};
+        for (int i = 0; i < 2; ++i)
+            for (const auto& ws : child_[i]->weight_specs()) specs.push_back({prefix(i) + ws.first, ws.second});
+        return specs;
+    }
+    void load(const PartTensors& t, Runtime& rt) override {
+        w_[0] = get(t, "left_out");
+        w_[1] = get(t, "right_out");
+        for (int i = 0; i < 2; ++i) {
+            PartTensors mine;
+            for (const auto& e : t)
+                if (e.first.rfind(prefix(i), 0) == 0) mine[e.first.substr(prefix(i).size())] = e.second;
+            child_[i]->load(mine, rt);
+        }
+    }
+    Tensor forward(const Tensor& x, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        Tensor result[2];
+        for (int i = 0; i < 2; ++i) {
+            LayerCache mine;
+            if (child_[i]->kv_need()) {
+                mine.kv = cache.kv;
+                mine.writes_kv = cache.writes_kv;
+            }
+            for (const auto& e : cache.states)
+                if (e.first.rfind(prefix(i), 0) == 0) mine.states[e.first.substr(prefix(i).size())] = e.second;
+            result[i] = child_[i]->forward(x, batch, mine, rt);
+            if (i == 1 && result[1].data == result[0].data) throw SpecError("normed_pair: both mixers answer in the same buffer");
+        }
+        Tensor out = rt.ws.buf("pair_out", rt.dtype, {x.shape[0], width_});
+        rt.ops.normed_mean(result[0], w_[0]->view, result[1], w_[1]->view, eps_, factor_, out);
+        return out;
+    }
+
+private:
+    static std::string prefix(int i) { return i == 0 ? "left." : "right."; }
+    long long width_ = 0;
+    float eps_ = 1e-6f, factor_ = 0.5f;
+    std::unique_ptr<Mixer> child_[2];
+    std::shared_ptr<DeviceTensor> w_[2];
+};
+
+// ---------------------------------------------------------------------------- gated linear attention
+// A recurrent mixer with a matrix of state per head and a decay per key channel:
+//     q = W_q h * dim^-1/2, k = W_k h (heads x dim), v = W_v h (heads x vdim)
+//     alpha = sigmoid(W_a2 (W_a1 h) + b_a2)^(1 / tau)      ("decay_rank": the width between a1 and a2)
+//     S <- diag(alpha) S + k v^T;   o = S^T q              per head, alpha on the rows of S
+// o is RMS-normed per head over vdim (weight [vdim] shared by the heads), the heads side by side
+// are multiplied by silu(W_g h) and go through W_o.  State per request: S [heads, dim, vdim], 32-bit;
+// decays, the recurrence and the norm are 32-bit.
+class GatedLinearAttention final : public Mixer {
+public:
+    explicit GatedLinearAttention(const PartSpec& s) : Mixer(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        shape_.heads = shape_.kv_heads = static_cast<int>(p.get_int("heads", 0));
+        shape_.dim = static_cast<int>(p.get_int("dim", 0));
+        shape_.vdim = static_cast<int>(p.get_int("vdim", shape_.dim));
+        shape_.taps = 1;
+        tau_ = static_cast<float>(p.get_double("tau", 1.0));
+        rank_ = p.get_int("decay_rank", 0);
+        eps_ = static_cast<float>(p.get_double("eps", 1e-6));
+        if (width_ <= 0 || shape_.heads <= 0 || shape_.dim <= 0 || shape_.vdim <= 0 || rank_ <= 0)
+            throw SpecError("gated_linear_attention: width, heads, dim, vdim and decay_rank must be positive");
+        if (!(tau_ > 0.f)) throw SpecError("gated_linear_attention: tau must be positive");
+    }
+    bool graph_safe() const override { return true; }
+    long long qk_width() const { return static_cast<long long>(shape_.heads) * shape_.dim; }
+    long long v_width() const { return static_cast<long long>(shape_.heads) * shape_.vdim; }
+    std::vector<StateNeed> state_needs() const override { return {StateNeed{"S", {shape_.heads, shape_.dim, shape_.vdim}, DType::F32}}; }
+    WeightSpecs weight_specs() const override {
+        return {{"q", matrix(qk_width(), width_)}, {"k", matrix(qk_width(), width_)}, {"v", matrix(v_width(), width_)},
+                {"g", matrix(v_width(), width_)},  {"a1", matrix(rank_, width_)},     {"a2", matrix(qk_width(), rank_)},
+                {"a2_bias", vec(qk_width())},      {"norm", vec(shape_.vdim, "around_one")}, {"o", matrix(width_, v_width())}};
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        const Stacked in = stack_projections({{get(t, "q"), false}, {get(t, "k"), false}, {get(t, "v"), false}, {get(t, "g"), false},
+                                              {get(t, "a1"), true}}, "gated_linear_attention");
+        w_in_ = in.weight;
+        col_k_ = in.at[1];
+        col_v_ = in.at[2];
+        col_g_ = in.at[3];
+        col_a_ = in.at[4];
+        a2_ = get(t, "a2");
+        a2_b_ = get(t, "a2_bias");
+        norm_ = get(t, "norm");
+        w_o_ = get(t, "o");
+    }
+    Tensor forward(const Tensor& x, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        const long long T = x.shape[0];
+        Tensor proj = rt.ws.buf("gla_proj", rt.dtype, {T, w_in_->view.shape[0]});
+        rt.ops.linear(x, w_in_->view, proj, nullptr, rt.ws);
+        Tensor z = rt.ws.buf("gla_decay_in", rt.dtype, {T, qk_width()});
+        rt.ops.linear(proj.cols(col_a_, rank_), a2_->view, z, nullptr, rt.ws);
+        Tensor qk = rt.ws.buf("gla_qk", DType::F32, {T, 2 * qk_width()}), v = rt.ws.buf("gla_v", DType::F32, {T, v_width()});
+        Tensor decay = rt.ws.buf("gla_decay", DType::F32, {T, qk_width()});
+        rt.ops.gla_prepare(proj.cols(0, qk_width()), proj.cols(col_k_, qk_width()), proj.cols(col_v_, v_width()), z, &a2_b_->view, tau_,
+                           static_cast<float>(1.0 / std::sqrt(static_cast<double>(shape_.dim))), qk, v, decay);
+        Tensor o = rt.ws.buf("gla_o", DType::F32, {T, v_width()});
+        rt.ops.channel_scan(qk, v, decay, nullptr, 0, cache.states.at("S"), o, shape_, batch);
+        Tensor gated = rt.ws.buf("gla_gated", rt.dtype, {T, v_width()});
+        rt.ops.delta_gated_norm(o, norm_->view, proj.cols(col_g_, v_width()), eps_, gated, shape_.heads, shape_.vdim, 0);
+        Tensor out = rt.ws.buf("gla_mixer_out", rt.dtype, {T, width_});
+        rt.ops.linear(gated, w_o_->view, out, nullptr, rt.ws);
+        return out;
+    }
+
+private:
+    long long width_ = 0, rank_ = 0, col_k_ = 0, col_v_ = 0, col_g_ = 0, col_a_ = 0;
+    Ops::DeltaShape shape_;
+    float tau_ = 1.f, eps_ = 1e-6f;
+    std::shared_ptr<DeviceTensor> w_in_, a2_, a2_b_, norm_, w_o_;
+};
+
+// ---------------------------------------------------------------------------- dense feed-forward with biases
+// mlp: W_down act(W_up x + b_up) + b_down; "activation": "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))))
+// or "relu2" (the square of relu); "bias": false leaves both biases out.
+class DenseMlp final : public FeedForward {
+public:
+    explicit DenseMlp(const PartSpec& s) : FeedForward(s), width_(s.params.get_int("width", 0)), ff_(s.params.get_int("ff", 0)) {
+        if (width_ <= 0 || ff_ <= 0) throw SpecError("mlp: width and ff must be positive");
+        const std::string act = s.params.get_string("activation", "gelu_tanh");
+        if (act != "gelu_tanh" && act != "relu2") throw SpecError("mlp: activation is 'gelu_tanh' or 'relu2', not '" + act + "'");
+        act_ = act == "relu2" ? 1 : 0;
+        bias_ = s.params.get_bool("bias", true);
+    }
+    bool graph_safe() const override { return true; }
+    WeightSpecs weight_specs() const override {
+        WeightSpecs specs{{"up", matrix(ff_, width_)}, {"down", matrix(width_, ff_)}};
+        if (bias_) {
+            specs.push_back({"up_bias", vec(ff_)});
+            specs.push_back({"down_bias", vec(width_)});
+        }
+        return specs;
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        w_up_ = get(t, "up");
+        w_down_ = get(t, "down");
+        b_up_ = maybe(t, "up_bias");
+        b_down_ = maybe(t, "down_bias");
+    }
+    Tensor forward(const Tensor& x, const StepBatch&, Runtime& rt) override {
+        const long long T = x.shape[0];
+        Tensor up = rt.ws.buf("mlp_up", rt.dtype, {T, ff_});
+        rt.ops.linear(x, w_up_->view, up, nullptr, rt.ws);
+        rt.ops.activation_bias(up, b_up_ ? &b_up_->view : nullptr, up, act_);
+        Tensor out = rt.ws.buf("ffn_out", rt.dtype, {T, width_});
+        rt.ops.linear(up, w_down_->view, out, b_down_ ? &b_down_->view : nullptr, rt.ws);
+        return out;
+    }
+
+private:
+    long long width_, ff_;
+    int act_ = 0;
+    bool bias_ = true;
+    std::shared_ptr<DeviceTensor> w_up_, w_down_, b_up_, b_down_;
+};
+
+// ---------------------------------------------------------------------------- a token input per layer
+// gated_table: with e = table[token][offset, offset + dim) (a table of "table_width" values a token that all
+// layers share, each reading its own columns), g = gelu_tanh(W_gate x) * e, y = W_proj g, and the stream
+// becomes x + y / sqrt(mean(y^2) + eps) * w with a plain weight.
+class GatedTableInput final : public TokenInput {
+public:
+    explicit GatedTableInput(const PartSpec& s) : TokenInput(s) {
+        const Json& p = s.params;
+        width_ = p.get_int("width", 0);
+        vocab_ = p.get_int("vocab", 0);
+        dim_ = p.get_int("dim", 0);
+        offset_ = p.get_int("offset", 0);
+        table_width_ = p.get_int("table_width", dim_);
+        eps_ = static_cast<float>(p.get_double("eps", 1e-6));
+        if (width_ <= 0 || vocab_ <= 0 || dim_ <= 0 || offset_ < 0 || offset_ + dim_ > table_width_)
+            throw SpecError("gated_table: width, vocab and dim must be positive and [offset, offset + dim) inside table_width");
+    }
+    bool graph_safe() const override { return true; }
+    WeightSpecs weight_specs() const override {
+        return {{"table", matrix(vocab_, table_width_)}, {"gate", matrix(dim_, width_)}, {"proj", matrix(width_, dim_)},
+                {"norm", vec(width_, "around_one")}};
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        table_ = get(t, "table");
+        gate_ = get(t, "gate");
+        proj_ = get(t, "proj");
+        norm_ = get(t, "norm");
+        post_.weight = norm_->view;
+        post_.eps = eps_;
+    }
+    void forward(const Tensor& h, const Tensor& h_copy, const StepBatch& batch, Runtime& rt) override {
+        const long long T = h.shape[0];
+        Tensor z = rt.ws.buf("token_input_z", rt.dtype, {T, dim_});
+        rt.ops.linear(h_copy, gate_->view, z, nullptr, rt.ws);
+        Tensor g = rt.ws.buf("token_input_g", rt.dtype, {T, dim_});
+        rt.ops.token_gate(z, table_->view, static_cast<int>(offset_), batch.token_ids, g);
+        Tensor y = rt.ws.buf("token_input_y", rt.dtype, {T, width_});
+        rt.ops.linear(g, proj_->view, y, nullptr, rt.ws);
+        rt.ops.norm_step(h, &y, &post_, nullptr, nullptr);
+    }
+
+private:
+    long long width_ = 0, vocab_ = 0, dim_ = 0, offset_ = 0, table_width_ = 0;
+    float eps_ = 1e-6f;
+    std::shared_ptr<DeviceTensor> table_, gate_, proj_, norm_;
+    Ops::NormParams post_;
+};
+
+// ---------------------------------------------------------------------------- a weighted sum over depth
+// weighted_history: behind run-order entry i the stream becomes sum_{j <= i + 1} w[j] X_j, X_0 the embedding's
+// rows and X_(j+1) the result of entry j before this mixing ("entries": how many results, i + 2).
+class WeightedHistory final : public DepthMix {
+public:
+    explicit WeightedHistory(const PartSpec& s) : DepthMix(s), entries_(static_cast<int>(s.params.get_int("entries", 0))) {
+        if (entries_ < 1) throw SpecError("weighted_history: entries must be positive");
+    }
+    bool graph_safe() const override { return true; }
+    int entries() const override { return entries_; }
+    WeightSpecs weight_specs() const override { return {{"weights", vec(entries_)}}; }
+    void load(const PartTensors& t, Runtime&) override { w_ = get(t, "weights"); }
+    void forward(const Tensor& history, const Tensor& h, Runtime& rt) override { rt.ops.depth_mix(history, h, w_->view, entries_); }
+
+private:
+    int entries_;
+    std::shared_ptr<DeviceTensor> w_;
+};
+
+// ---------------------------------------------------------------------------- both sub-layers from one norm
+// parallel: h += mixer(norm(h)) + ffn(norm(h)): one norm, both sub-layers read its output, one sum into
+// the 32-bit stream.  A feed-forward of kind "none" is left out.
+class ParallelBlock final : public Block {
+public:
+    explicit ParallelBlock(const LayerSpec& layer)
+        : norm_(build_as<Norm>("norm", layer.mixer_norm)), mixer_(build_as<Mixer>("mixer", layer.mixer)),
+          has_ffn_(layer.ffn.kind != "none" && !layer.ffn.kind.empty()) {
+        if (has_ffn_) ffn_ = build_as<FeedForward>("ffn", layer.ffn);
+    }
+    std::vector<std::pair<std::string, Part*>> parts() override {
+        std::vector<std::pair<std::string, Part*>> out{{"mixer_norm", norm_.get()}, {"mixer", mixer_.get()}};
+        if (has_ffn_) out.emplace_back("ffn", ffn_.get());
+        return out;
+    }
+    Mixer& mixer() override { return *mixer_; }
+    Tensor forward(const Tensor& h, const Tensor& delta, const StepBatch& batch, const LayerCache& cache, Runtime& rt) override {
+        const long long T = h.shape[0], width = h.shape[1];
+        rt.stream_stat_blocks = 0;
+        rt.stream_has_bf16 = false;
+        Tensor normed = rt.ws.buf("normed", rt.dtype, {T, width});
+        norm_->forward(h, normed, rt, delta.defined() ? &delta : nullptr, nullptr);
+        Tensor mixed = mixer_->forward(normed, batch, cache, rt);
+        rt.mark("mixer " + mixer_->spec.kind);
+        Tensor fed;
+        if (has_ffn_) {
+            fed = ffn_->forward(normed, batch, rt);
+            rt.mark("ffn " + ffn_->spec.kind);
+        }
+        // the sum into the stream, and the stream's new rows in the run's dtype for whoever reads them next
+        Tensor copy = rt.ws.buf("stream_copy", rt.dtype, {T, width});
+        rt.ops.residual_sum(h, mixed, has_ffn_ ? &fed : nullptr, &copy);
+        rt.stream_copy = copy;
+        return Tensor();
+    }
+
+private:
+    std::unique_ptr<Norm> norm_;
+    std::unique_ptr<Mixer> mixer_;
+    bool has_ffn_;
+    std::unique_ptr<FeedForward> ffn_;
+};
+
 template <typename T>
 PartFactory factory_of() {
     return [](const PartSpec& s) { return std::unique_ptr<Part>(new T(s)); };
@@ -1439,6 +2004,13 @@ void register_builtin_parts() {
     r.parts["mixer"]["sigmoid_attention"] = factory_of<SigmoidAttention>();
     r.parts["mixer"]["gated_delta_rule"] = factory_of<GatedDeltaRule>();
     r.parts["reinjection"]["linear_concat"] = factory_of<LinearReinjection>();
+    r.parts["mixer"]["biased_attention"] = factory_of<BiasedAttention>();
+    r.parts["mixer"]["linear_recurrent_unit"] = factory_of<LinearRecurrentUnit>();
+    r.parts["mixer"]["normed_pair"] = factory_of<NormedPair>();
+    r.parts["mixer"]["gated_linear_attention"] = factory_of<GatedLinearAttention>();
+    r.parts["ffn"]["mlp"] = factory_of<DenseMlp>();
+    r.parts["token_input"]["gated_table"] = factory_of<GatedTableInput>();
+    r.parts["depth_mix"]["weighted_history"] = factory_of<WeightedHistory>();
     r.parts["mixer"]["none"] = factory_of<NoMixer>();
     r.parts["ffn"]["swiglu"] = factory_of<SwiGlu>();
     r.parts["ffn"]["routed_experts"] = factory_of<RoutedExperts>();
@@ -1449,6 +2021,7 @@ void register_builtin_parts() {
     r.parts["head"]["linear_head"] = factory_of<LinearHead>();
     r.parts["head"]["hidden"] = factory_of<HiddenHead>();
     r.blocks["pre_norm"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new PreNormBlock(layer)); };
+    r.blocks["parallel"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new ParallelBlock(layer)); };
     r.blocks["sandwich_norm"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new SandwichBlock(layer)); };
     r.blocks["hyper_connections"] = [](const LayerSpec& layer) { return std::unique_ptr<Block>(new HyperBlock(layer)); };
 }

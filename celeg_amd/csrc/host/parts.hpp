@@ -75,6 +75,25 @@ public:
     virtual void forward(const Tensor& h, const Tensor& x0, Runtime& rt) = 0;
 };
 
+// What the rows' token ids add to the residual stream after a layer's sub-layers.
+class TokenInput : public Part {
+public:
+    using Part::Part;
+    // h [T, width] 32-bit, the stream, is added to; h_copy holds the same rows in the run's dtype
+    virtual void forward(const Tensor& h, const Tensor& h_copy, const StepBatch& batch, Runtime& rt) = 0;
+};
+
+// How the stream behind an entry of the run order is mixed from the results of all entries so far.
+class DepthMix : public Part {
+public:
+    using Part::Part;
+    // how many results it mixes: the embedding's rows and those of the entries up to its own
+    virtual int entries() const = 0;
+    // history [>= entries, T, width] 32-bit holds the earlier results; h, this entry's result, is
+    // recorded as the last of them and replaced by the mixture
+    virtual void forward(const Tensor& history, const Tensor& h, Runtime& rt) = 0;
+};
+
 class PositionEncoding : public Part {
 public:
     using Part::Part;
@@ -143,7 +162,7 @@ public:
 using PartFactory = std::function<std::unique_ptr<Part>(const PartSpec&)>;
 using BlockFactory = std::function<std::unique_ptr<Block>(const LayerSpec&)>;
 
-// role: norm, mixer, ffn, position, embedding, head, link, reinjection
+// role: norm, mixer, ffn, position, embedding, head, link, reinjection, token_input, depth_mix
 void register_part(const std::string& role, const std::string& kind, PartFactory factory, bool replace = false);
 void register_block(const std::string& arrangement, BlockFactory factory, bool replace = false);
 std::unique_ptr<Part> build_part(const std::string& role, const PartSpec& spec);

@@ -15,7 +15,10 @@
 //           "arrangement": "pre_norm"}; an arrangement that joins a sub-layer to the residual
 //           stream by a part of its own names them as "mixer_link" and "ffn_link"; one that norms
 //           a sub-layer's output before the addition names those norms "mixer_post_norm" and
-//           "ffn_post_norm"
+//           "ffn_post_norm"; a layer may name a "token_input" (a part that adds something made from the
+//           rows' token ids to the stream after the sub-layers) and a "depth_mix" (a part that replaces
+//           the stream behind the layer by a mixture of the results of all entries of the run order so
+//           far, the embedding's rows first)
 //   model: {"architecture", "vocab_size", "hidden_size", "max_context", "streams" (residual
 //           streams per row, 1 if absent), "embedding": part,
 //           "layers": [layer], "order": [{"layer": i, "kv_from": j or null, "reinject": bool}],
@@ -85,6 +88,9 @@ struct LayerSpec {
     PartSpec mixer_link, ffn_link;
     // norms of the sub-layers' outputs, for arrangements that norm before and after (kind empty: none)
     PartSpec mixer_post_norm, ffn_post_norm;
+    // what the rows' token ids add to the stream after the sub-layers, and how the stream behind the
+    // layer is mixed from the results of the entries run so far (kind empty: none)
+    PartSpec token_input, depth_mix;
     std::string arrangement = "pre_norm";
 };
 
@@ -140,6 +146,8 @@ struct ModelSpec {
             if (!l.ffn_link.kind.empty()) lj.set("ffn_link", l.ffn_link.to_json());
             if (!l.mixer_post_norm.kind.empty()) lj.set("mixer_post_norm", l.mixer_post_norm.to_json());
             if (!l.ffn_post_norm.kind.empty()) lj.set("ffn_post_norm", l.ffn_post_norm.to_json());
+            if (!l.token_input.kind.empty()) lj.set("token_input", l.token_input.to_json());
+            if (!l.depth_mix.kind.empty()) lj.set("depth_mix", l.depth_mix.to_json());
             ls.push(lj);
         }
         Json ord = Json::array();
@@ -181,6 +189,8 @@ struct ModelSpec {
             if (!l["ffn_link"].is_null()) ls.ffn_link = PartSpec::from_json(l["ffn_link"], where + ".ffn_link");
             if (!l["mixer_post_norm"].is_null()) ls.mixer_post_norm = PartSpec::from_json(l["mixer_post_norm"], where + ".mixer_post_norm");
             if (!l["ffn_post_norm"].is_null()) ls.ffn_post_norm = PartSpec::from_json(l["ffn_post_norm"], where + ".ffn_post_norm");
+            if (!l["token_input"].is_null()) ls.token_input = PartSpec::from_json(l["token_input"], where + ".token_input");
+            if (!l["depth_mix"].is_null()) ls.depth_mix = PartSpec::from_json(l["depth_mix"], where + ".depth_mix");
             ls.arrangement = l.get_string("arrangement", "pre_norm");
             m.layers.push_back(std::move(ls));
         }

@@ -187,10 +187,11 @@ __global__ void moe_gather_kernel(const T* __restrict__ x, const int* __restrict
 
 // ---------------------------------------------------------------- product over the tiles
 // w: [E, N, K]; a: [n, K]; out: [n, N].  gated: w holds, per expert, N gate rows then N up rows, and
-// out = silu(a gate^T) * (a up^T) (the two sums rounded to T first, as where they are tensors).
+// out = silu(a gate^T) * (a up^T) (the two sums rounded to T first, as where they are tensors).  Not gated, with
+// act 1: the square of relu of the sum (rounded to T first); act 0: the sum itself.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ a, const T* __restrict__ w,
-                                                          T* __restrict__ out, int N, int K, int gated,
+                                                          T* __restrict__ out, int N, int K, int gated, int act,
                                                           const int* __restrict__ offsets,
                                                           const int* __restrict__ tile_expert,
                                                           const int* __restrict__ tile_row0,
@@ -219,6 +220,9 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
             if (gated) {
                 const float g = to_float(from_float<T>(v)), u = to_float(from_float<T>(ups.v[i][j]));
                 v = (g / (1.0f + expf(-g))) * u;
+            } else if (act == 1) {
+                const float z = fmaxf(to_float(from_float<T>(v)), 0.f);
+                v = z * z;
             }
             out[static_cast<size_t>(row0 + r) * N + col0 + c] = from_float<T>(v);
         }
@@ -231,7 +235,7 @@ __global__ __launch_bounds__(256) void moe_product_kernel(const T* __restrict__ 
 // workgroups pull the weights).
 template <bool GATED, int MOE_CT>
 __global__ __launch_bounds__(256, 2) void moe_product_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w,
-                                                                  __bf16* __restrict__ out, int N, int K,
+                                                                  __bf16* __restrict__ out, int N, int K, int act,
                                                                   const int* __restrict__ offsets,
                                                                   const int* __restrict__ tile_expert,
                                                                   const int* __restrict__ tile_row0,
@@ -272,6 +276,9 @@ __global__ __launch_bounds__(256, 2) void moe_product_mfma_kernel(const __bf16* 
                     const float g = static_cast<float>(static_cast<__bf16>(x));
                     const float u = static_cast<float>(static_cast<__bf16>(sums[S - 1][ct][rt][r]));
                     x = (g / (1.0f + expf(-g))) * u;
+                } else if (act == 1) {
+                    const float z = fmaxf(static_cast<float>(static_cast<__bf16>(x)), 0.f);
+                    x = z * z;
                 }
                 v[r] = static_cast<__bf16>(x);
             }
@@ -349,7 +356,7 @@ extern "C" int celeg_moe_gather(const void* x, int dtype, const int* entry_at, c
     return CELEG_LAUNCH_RESULT();
 }
 
-extern "C" int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated,
+extern "C" int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated, int act,
                                  const int* offsets, const int* tile_expert, const int* tile_row0, const int* n_tiles,
                                  int max_tiles, int tile_rows, int wide, hipStream_t stream) {
     if (max_tiles <= 0) return 0;
@@ -359,7 +366,7 @@ extern "C" int celeg_moe_product(const void* a, const void* w, void* out, int dt
         dim3 grid(max_tiles, (N + MR_COLS * ct - 1) / (MR_COLS * ct));
 #define MOE_GO(GATED, CT)                                                                                                       \
     hipLaunchKernelGGL((moe_product_mfma_kernel<GATED, CT>), grid, dim3(256), 0, stream, static_cast<const __bf16*>(a),         \
-                       static_cast<const __bf16*>(w), static_cast<__bf16*>(out), N, K, offsets, tile_expert, tile_row0, n_tiles)
+                       static_cast<const __bf16*>(w), static_cast<__bf16*>(out), N, K, act, offsets, tile_expert, tile_row0, n_tiles)
         if (gated && wide) MOE_GO(true, 2);
         else if (gated) MOE_GO(true, 1);
         else if (wide) MOE_GO(false, 4);
@@ -371,11 +378,11 @@ extern "C" int celeg_moe_product(const void* a, const void* w, void* out, int dt
     dim3 grid(max_tiles, (N + SG_COLS - 1) / SG_COLS);
     if (dtype == CELEG_F32)
         hipLaunchKernelGGL(moe_product_kernel<float>, grid, dim3(256), 0, stream, static_cast<const float*>(a),
-                           static_cast<const float*>(w), static_cast<float*>(out), N, K, gated, offsets, tile_expert,
+                           static_cast<const float*>(w), static_cast<float*>(out), N, K, gated, act, offsets, tile_expert,
                            tile_row0, n_tiles);
     else
         hipLaunchKernelGGL(moe_product_kernel<bf16>, grid, dim3(256), 0, stream, static_cast<const bf16*>(a),
-                           static_cast<const bf16*>(w), static_cast<bf16*>(out), N, K, gated, offsets, tile_expert,
+                           static_cast<const bf16*>(w), static_cast<bf16*>(out), N, K, gated, act, offsets, tile_expert,
                            tile_row0, n_tiles);
     return CELEG_LAUNCH_RESULT();
 }
