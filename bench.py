@@ -159,6 +159,44 @@ KIFETAR_SHAPES = {
            lfm2_shape(2048, 32, 8, 4096, KIFETAR_ATTENTION, 8, 8192)),
 }
 
+# Kivorax beside Kifetar, the closest existing design (attention layers and matrix-state recurrences
+# from the same parts): attention where Kivorax has its pair of attention and recurrent unit, the delta
+# rule with a decay per head where Kivorax has the delta rule with a decay per key channel or gated
+# linear attention; same width, heads, head sizes and vocabulary, a dense feed-forward as wide as the
+# experts a token uses together.
+def kivorax_shape(width, pattern, heads, kv_heads, dim, vdim, inner, blocks, d_heads, d_kv_heads, d_dim, d_vdim, experts, top, ff,
+                  side=64, vocab=65536):
+    moe = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    pair = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5,
+                     "q_temp": {"coef": 0.1, "every": 512}},
+            "right": {"width": inner, "blocks": blocks, "conv": 4}}
+    delta = {"heads": d_heads, "kv_heads": d_kv_heads, "dim": d_dim, "vdim": d_vdim, "conv": 4, "decay_rank": 64, "gate_rank": 64}
+    gla = {"heads": d_heads, "dim": d_dim, "vdim": d_vdim, "tau": 16.0, "decay_rank": 64}
+    kinds = {"p": ("parallel", pair), "d": ("channel_delta", delta), "g": ("gla", gla)}
+    layers = [{"type": kinds[c][0], "mixer": kinds[c][1], "mlp": moe} for c in pattern]
+    layers[0]["mlp"] = {"kind": "dense", "ff": ff * top}
+    return {"architecture": "Kivorax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "token_side": {"dim": side}, "max_context": 8192, "layers": layers}
+
+
+def kifetar_beside(width, pattern, heads, kv_heads, dim, d_heads, d_kv_heads, d_dim, d_vdim, ff, vocab=65536):
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                 "rot": {"base": 500000.0, "dims": dim // 2}}
+    delta = {"heads": d_heads, "kv_heads": d_kv_heads, "dim": d_dim, "vdim": d_vdim, "conv": 4}
+    mlp = {"kind": "dense", "ff": ff}
+    return {"architecture": "Kifetar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "max_context": 8192,
+            "layers": [{"type": "attention", "mixer": attention, "mlp": mlp} if kind == "p" else
+                       {"type": "delta", "mixer": delta, "mlp": mlp} for kind in pattern]}
+
+
+KIVORAX_PATTERN = "pddgpddg"
+KIVORAX_SHAPES = {
+    "1k": (kivorax_shape(1024, KIVORAX_PATTERN, 16, 8, 64, 64, 1024, 8, 16, 8, 64, 64, 16, 2, 1024),
+           kifetar_beside(1024, KIVORAX_PATTERN, 16, 8, 64, 16, 8, 64, 64, 2048)),
+    "2k": (kivorax_shape(2048, KIVORAX_PATTERN, 16, 8, 128, 128, 2048, 8, 16, 8, 128, 128, 32, 4, 1024),
+           kifetar_beside(2048, KIVORAX_PATTERN, 16, 8, 128, 16, 8, 128, 128, 4096)),
+}
+
 DESIGN_SHAPES = {
     "1k": (regipel_shape(1024, 8, 16, 64, 32, 64, 256, 16, 2, 1024), lfm2_shape(1024, 16, 8, 2048, set(range(8)), 8, 8192)),
     "2k": (regipel_shape(2048, 8, 16, 128, 64, 128, 512, 32, 4, 1024), lfm2_shape(2048, 32, 8, 4096, set(range(8)), 8, 8192)),
@@ -174,13 +212,14 @@ def design(shapes, steps: int, warmup: int, batch: int, layers: int = 0, profile
     from celeg_amd.weights import write_random_model
     out = {}
     for shape in shapes:
-        table, beside = (KIFETAR_SHAPES, "lfm2_hybrid") if which == "kifetar" else (DESIGN_SHAPES, "lfm2_attention")
+        table, beside = {"kifetar": (KIFETAR_SHAPES, "lfm2_hybrid"), "kivorax": (KIVORAX_SHAPES, "kifetar_beside"),
+                         "regipel": (DESIGN_SHAPES, "lfm2_attention")}[which]
         for label, cfg in zip((which, beside), table[shape]):
             if profile_only and label != profile_only:
                 continue
             cfg = json.loads(json.dumps(cfg))
             if layers:
-                if label == which:
+                if "layers" in cfg:
                     cfg["layers"] = cfg["layers"][:layers]
                 else:
                     cfg.update(num_hidden_layers=layers, layer_types=cfg["layer_types"][:layers])
@@ -204,7 +243,8 @@ def design(shapes, steps: int, warmup: int, batch: int, layers: int = 0, profile
                 "weights": lm.native.info["weights"], "kv_bytes_per_token": lm.native.info["kv_bytes_per_token"],
                 "layers": len(lm.native.info["spec"]["order"])}
             engine.close()
-    title = "Kifetar beside LFM2 convolution and attention layers" if which == "kifetar" else "Regipel beside LFM2 attention layers"
+    title = {"kifetar": "Kifetar beside LFM2 convolution and attention layers", "regipel": "Regipel beside LFM2 attention layers",
+             "kivorax": "Kivorax beside Kifetar attention and delta-rule layers"}[which]
     print(json.dumps({"metric": title + " at equal size: prefill tok/s @ 2048 tokens, "
                                 f"decode tok/s @ batch {batch}, context 2048 (bf16, random weights)",
                       "phase": "design", "design": which, "batch": batch, "steps": steps, "warmup": warmup, "dtype": "bf16",
@@ -234,15 +274,15 @@ def main() -> int:
                          "(default 2048, the headline's); with --phase prefill: tokens of the same "
                          "prompt that the cache holds before the measured portion of 2,048 (default 0)")
     ap.add_argument("--design-shape", default="1k,2k", help="with --phase design: which sizes (1k, 2k)")
-    ap.add_argument("--design", default="regipel", choices=["regipel", "kifetar"],
+    ap.add_argument("--design", default="regipel", choices=["regipel", "kifetar", "kivorax"],
                     help="with --phase design: which design is measured beside its closest LFM2 shape")
-    ap.add_argument("--design-model", default="", choices=["", "regipel", "lfm2_attention", "kifetar", "lfm2_hybrid"],
+    ap.add_argument("--design-model", default="", choices=["", "regipel", "lfm2_attention", "kifetar", "lfm2_hybrid", "kivorax", "kifetar_beside"],
                     help="with --phase design: only this model (for profiling)")
     ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve", "design"], default="all",
                     help="for profiling: run only the prefill measurement, or only the batch-8 "
                          "decode measurement (the line printed then holds only that part); "
                          "serve: the whole engine on the serving workload of --shape; design: the "
-                         "Regipel design beside LFM2 attention layers at equal size")
+                         "design named by --design beside its closest existing model at equal size")
     ap.add_argument("--knob", action="append", default=[], metavar="NAME=VALUE",
                     help="set a knob of the step function or the kernels' dispatch before measuring "
                          "(tuning runs; the names are those of celeg_model_knobs)")

@@ -1555,7 +1555,7 @@ public:
         WeightSpecs specs{{"q", matrix(q_width(), width_)}, {"k", matrix(k_width(), width_)}, {"v", matrix(v_width(), width_)},
                           {"o", matrix(width_, o_width())}};
         if (distance_bias_) {
-            specs.push_back({"r1", vec(shape_.heads)});
+            specs.push_back({"r1", vec(shape_.heads, "around_one")});
             specs.push_back({"r2", vec(shape_.heads, "around_one")});
         }
         if (gated_) specs.push_back({"g", matrix(o_width(), width_)});
@@ -1933,7 +1933,7 @@ public:
     }
     bool graph_safe() const override { return true; }
     int entries() const override { return entries_; }
-    WeightSpecs weight_specs() const override { return {{"weights", vec(entries_)}}; }
+    WeightSpecs weight_specs() const override { return {{"weights", vec(entries_, "around_one")}}; }
     void load(const PartTensors& t, Runtime&) override { w_ = get(t, "weights"); }
     void forward(const Tensor& history, const Tensor& h, Runtime& rt) override { rt.ops.depth_mix(history, h, w_->view, entries_); }
 
