@@ -185,21 +185,6 @@ __global__ __launch_bounds__(CELEG_WAVE) void delta_pairs_kernel(const float* __
     }
 }
 
-// The sum of v over every group of W neighbouring lanes (1 to 16), in all of them, by the vector
-// unit's cross-lane modifiers: lanes swapped in pairs and in pairs of pairs, then the halves of 8
-// and of 16 mirrored.  Both sides of every exchange add the same two numbers, so the lanes agree.
-template <int W>
-__device__ __forceinline__ float lanes_sum(float v) {
-    auto across = [](float x, auto ctrl) {
-        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, false));
-    };
-    if (W >= 2) v += across(v, std::integral_constant<int, 0xB1>{});
-    if (W >= 4) v += across(v, std::integral_constant<int, 0x4E>{});
-    if (W >= 8) v += across(v, std::integral_constant<int, 0x141>{});
-    if (W >= 16) v += across(v, std::integral_constant<int, 0x140>{});
-    return v;
-}
-
 // The same recurrence with S in registers, for dim = DL * DPL: DL neighbouring lanes share a column
 // of S, each holding DPL of its values, so a wavefront owns 64 / DL columns and the sums over dim
 // meet by log2(DL) exchanges between neighbours.  (Few values a lane: a token's passes over the

@@ -607,7 +607,7 @@ const std::vector<Knob>& knobs() {
         OPS_INT(attention_decode_whole), OPS_BOOL(use_blaslt), OPS_INT(attention_rows_per_tile), OPS_INT(attention_rows_form),
         OPS_BOOL(attention_general), OPS_BOOL(use_rope_table), OPS_BOOL(use_argmax_parts), OPS_BOOL(use_head_argmax), OPS_BOOL(decode_parts_fill), OPS_BOOL(use_sliced),
         OPS_BOOL(use_rows_kernel), OPS_BOOL(use_tiles), OPS_BOOL(use_qkv_tail), OPS_BOOL(use_fresh_decode), OPS_INT(rows_kernel_min_rows), OPS_INT(tiles_min_rows),
-        OPS_INT(fused_linear_shape), OPS_BOOL(use_latent_mfma), OPS_BOOL(delta_general), OPS_BOOL(delta_pairs), OPS_BOOL(use_sigmoid_mfma), OPS_INT(sigmoid_rows_form), OPS_BOOL(use_moe_mfma), OPS_BOOL(use_router_kernel), OPS_INT(latent_decode_workgroups), OPS_INT(latent_decode_min_blocks),
+        OPS_INT(fused_linear_shape), OPS_BOOL(use_latent_mfma), OPS_BOOL(delta_general), OPS_BOOL(delta_pairs), OPS_BOOL(use_sigmoid_mfma), OPS_INT(sigmoid_rows_form), OPS_BOOL(use_biased_mfma), OPS_INT(biased_rows_form), OPS_BOOL(use_moe_mfma), OPS_BOOL(use_router_kernel), OPS_INT(latent_decode_workgroups), OPS_INT(latent_decode_min_blocks),
         {"decode_parts_few", [](LoadedModel& m) { return m.rt->ops.decode_part_thresholds[0]; }, [](LoadedModel& m, int v) { m.rt->ops.decode_part_thresholds[0] = v; }},
         {"decode_parts_some", [](LoadedModel& m) { return m.rt->ops.decode_part_thresholds[1]; }, [](LoadedModel& m, int v) { m.rt->ops.decode_part_thresholds[1] = v; }},
     };

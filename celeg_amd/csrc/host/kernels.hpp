@@ -189,6 +189,13 @@ int celeg_biased_attention(const void* q, int ldq, int dtype, const void* k_pool
                            const void* gate, int ldg, void* out, int ldo, int n_tokens, int q_heads, int kv_heads, int head_dim,
                            int v_dim, int page_tokens, int n_layers, int layer, float scale, float coef, int every, int window,
                            hipStream_t stream);
+// biased_attention_fast.hip
+int celeg_biased_attention_fast_ok(int head_dim, int v_dim);
+int celeg_biased_attention_fast(int form, const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table, int table_stride,
+                                const int* cu_seqlens, const int* seq_slot, const int* seq_start, int n_seqs, int max_tiles,
+                                const float* r1, const float* r2, const void* gate, int ldg, void* out, int ldo, int q_heads,
+                                int kv_heads, int head_dim, int v_dim, int page_tokens, int n_layers, int layer, float scale, float coef,
+                                int every, int window, hipStream_t stream);
 // linear_scan.hip
 int celeg_lru_gates(const void* x, int ldx, int dtype, const float* conv_w, const float* conv_b, const float* ra_t, const float* ra_b,
                     const float* ri_t, const float* ri_b, const float* lam, const float* conv_state, size_t state_stride,
@@ -203,5 +210,5 @@ int celeg_gla_prepare(const void* q, int ldq, const void* k, int ldk, const void
                       int qk_cols, int v_cols, hipStream_t stream);
 int celeg_channel_scan(const float* qk, const float* v, const float* decay, const float* beta, int ld_beta, float* state,
                        size_t state_stride, const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G, int H, int D,
-                       int V, hipStream_t stream);
+                       int V, int general, hipStream_t stream);
 }

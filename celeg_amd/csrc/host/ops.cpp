@@ -60,6 +60,7 @@ const char* path_name(Path p) {
         case Path::AttentionLatentDecode: return "attention_latent_decode";
         case Path::AttentionBiased: return "attention_biased";
         case Path::AttentionBiasedRows: return "attention_biased_rows";
+        case Path::AttentionBiasedDecode: return "attention_biased_decode";
         case Path::ChannelScan: return "channel_scan";
         case Path::LinearRecurrentUnit: return "linear_recurrent_unit";
         case Path::RoutedExperts: return "routed_experts";
@@ -923,7 +924,7 @@ void Ops::channel_scan(const Tensor& qk, const Tensor& v, const Tensor& decay, c
     took(Path::ChannelScan);
     kernel_check(celeg_channel_scan(qk.as<float>(), v.as<float>(), decay.as<float>(), beta, beta_ld, state.as<float>(),
                                     static_cast<size_t>(state.stride[0]), batch.cu_seqlens, batch.seq_slot, out.as<float>(),
-                                    batch.n_seqs, s.kv_heads, s.heads, s.dim, s.vdim, stream), "channel_scan");
+                                    batch.n_seqs, s.kv_heads, s.heads, s.dim, s.vdim, delta_general ? 1 : 0, stream), "channel_scan");
 }
 
 // ---------------------------------------------------------------------------- linear recurrent unit
@@ -1030,6 +1031,24 @@ void Ops::biased_attention(const Tensor& q, const Tensor& out, const ScoreShape&
     }
     (void)ws;
     took(Path::AttentionBiased);
+    const int ldq = rows_of(q, "q"), ldo = rows_of(out, "out"), ldg = gate ? rows_of(*gate, "gate") : 0;
+    auto aligned = [](const void* p, uintptr_t bytes) { return (reinterpret_cast<uintptr_t>(p) & (bytes - 1)) == 0; };
+    if (q.dtype == DType::BF16 && use_biased_mfma && !attention_general && celeg_biased_attention_fast_ok(s.head_dim, s.v_dim) &&
+        kv.page_tokens >= 8 && (kv.page_tokens & (kv.page_tokens - 1)) == 0 && ldq % 8 == 0 && ldo % 4 == 0 && ldg % 4 == 0 &&
+        aligned(q.data, 16) && aligned(out.data, 8) && (!gate || aligned(gate->data, 8))) {
+        // portions of prompts: tiles of 64 rows that share their staged keys; single tokens and short
+        // portions: tiles of 16 rows whose key blocks the wavefronts take in turn.  At most one
+        // partly filled tile per request.
+        const int form = biased_rows_form >= 0 ? biased_rows_form : (batch.max_seg_len > 16 ? 1 : 0);
+        const int max_tiles = static_cast<int>(T) / (form == 1 ? 64 : 16) + batch.n_seqs;
+        took(batch.decode_only ? Path::AttentionBiasedDecode : Path::AttentionBiasedRows);
+        kernel_check(celeg_biased_attention_fast(form, q.data, ldq, kv.k, kv.v, kv.table, kv.table_stride, batch.cu_seqlens, batch.seq_slot,
+                                                 batch.seq_start, batch.n_seqs, max_tiles, r1 ? r1->as<float>() : nullptr,
+                                                 r2 ? r2->as<float>() : nullptr, gate ? gate->data : nullptr, ldg, out.data, ldo, s.heads,
+                                                 s.kv_heads, s.head_dim, s.v_dim, kv.page_tokens, kv.n_layers, kv.layer, s.scale, s.coef,
+                                                 s.every, s.window, stream), "biased attention (bfloat16, matrix cores)");
+        return;
+    }
     kernel_check(celeg_biased_attention(q.data, rows_of(q, "q"), dt(q, "q"), kv.k, kv.v, kv.table, kv.table_stride, batch.token_slot,
                                         batch.positions, r1 ? r1->as<float>() : nullptr, r2 ? r2->as<float>() : nullptr,
                                         gate ? gate->data : nullptr, gate ? rows_of(*gate, "gate") : 0, out.data, rows_of(out, "out"),

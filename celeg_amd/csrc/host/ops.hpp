@@ -102,7 +102,7 @@ struct StepPrologue {
 // graph records; a replay counts nothing): what tests and tools ask to see that a size took the
 // path it was meant to take.
 enum class Path : int {
-    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionSigmoid, AttentionSigmoidRows, AttentionSigmoidDecode, DeltaRule, AttentionLatent, AttentionLatentRows, AttentionLatentDecode, AttentionBiased, AttentionBiasedRows, ChannelScan, LinearRecurrentUnit, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
+    AttentionDecode = 0, AttentionDecodeFresh, AttentionRows, AttentionGeneral, AttentionSigmoid, AttentionSigmoidRows, AttentionSigmoidDecode, DeltaRule, AttentionLatent, AttentionLatentRows, AttentionLatentDecode, AttentionBiased, AttentionBiasedRows, AttentionBiasedDecode, ChannelScan, LinearRecurrentUnit, RoutedExperts, LinearF32, LinearLibrary, LinearStandIn,
     FusedSliced, FusedRows, FusedStaged, Tiled, TiledQkv, ArgmaxMerged, Count
 };
 const char* path_name(Path p);
@@ -127,6 +127,7 @@ public:
     bool delta_pairs = true;             // the recurrence in registers takes whole blocks of rows two tokens at a time
     bool use_sigmoid_mfma = true;        // bfloat16 attention with sigmoid weights on the matrix cores
     bool use_biased_mfma = true;         // bfloat16 attention with a distance bias on the matrix cores
+    int biased_rows_form = -1;           // likewise for the attention with a distance bias
     int sigmoid_rows_form = -1;          // -1: by the step's longest portion; 0 tiles of 16 rows, 1 tiles of 64 rows
     bool use_router_kernel = true;       // the router's product inside the routing kernel
     bool use_moe_mfma = true;            // bfloat16 products of routed experts and per-head matrices on the matrix cores

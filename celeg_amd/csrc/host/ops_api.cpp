@@ -162,6 +162,8 @@ void set_knobs(Ops& ops, const Json& knobs) {
         else if (name == "delta_pairs") ops.delta_pairs = v != 0;
         else if (name == "sigmoid_rows_form") ops.sigmoid_rows_form = static_cast<int>(v);
         else if (name == "use_sigmoid_mfma") ops.use_sigmoid_mfma = v != 0;
+        else if (name == "use_biased_mfma") ops.use_biased_mfma = v != 0;
+        else if (name == "biased_rows_form") ops.biased_rows_form = static_cast<int>(v);
         else if (name == "use_argmax_parts") ops.use_argmax_parts = v != 0;
         else if (name == "use_head_argmax") ops.use_head_argmax = v != 0;
         else if (name == "decode_parts_fill") ops.decode_parts_fill = v != 0;

@@ -217,6 +217,115 @@ __global__ __launch_bounds__(CELEG_WAVE) void channel_scan_kernel(
     }
 }
 
+// The same recurrence for dim = DL * DPL (DPL a multiple of 4): DL neighbouring lanes share a column
+// of S, each holding DPL neighbouring values of it, so the sums over dim meet by log2(DL) exchanges
+// through the vector unit's cross-lane modifiers.  A request's rows are taken in blocks of TB
+// tokens whose q, k and decays are staged in LDS (asked for from memory while the block before is
+// computed) and whose values sit in registers; a token's steps wait for LDS, never for memory.
+// Tokens are taken one at a time in every block, so the cut of a prompt into steps changes no bit.
+template <int DL, int DPL, bool BETA>
+__global__ __launch_bounds__(CELEG_WAVE) void channel_scan_block_kernel(
+    const float* __restrict__ qk, const float* __restrict__ v, const float* __restrict__ decay, const float* __restrict__ beta,
+    int ld_beta, float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ seq_slot, float* __restrict__ out, int G, int H, int V) {
+    constexpr int D = DL * DPL, NC = DPL / 4, CPW = CELEG_WAVE / DL, TB = D <= 64 ? 16 : 8, ROW = 3 * D;
+    constexpr int PER_LANE = TB * ROW / CELEG_WAVE;
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) float rows_s[TB * ROW];
+    __shared__ float beta_s[TB];
+    const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int sub = lane % DL, j = blockIdx.z * CPW + lane / DL;
+    const bool live = j < V;
+    const int jj = live ? j : V - 1;          // idle lanes repeat the last column and store nothing
+    const int g = h / (H / G);
+    const int row0 = cu_seqlens[s], n = cu_seqlens[s + 1] - row0;
+    if (n <= 0) return;
+    float* mine = state + static_cast<size_t>(seq_slot[s]) * state_stride + static_cast<size_t>(h) * D * V;
+    float S[DPL];
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) S[i] = mine[static_cast<size_t>(sub * DPL + i) * V + jj];
+    const size_t ldqk = static_cast<size_t>(2) * G * D, ldv = static_cast<size_t>(H) * V, ldd = static_cast<size_t>(H) * D;
+    float pre[PER_LANE], pre_v[TB], pre_b = 1.f;
+    auto fetch = [&](int block) __attribute__((always_inline)) {
+        const int t0 = block * TB;
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) {
+            const int e = lane + CELEG_WAVE * i, tt = e / ROW, x = e % ROW;
+            pre[i] = 0.f;
+            if (t0 + tt < n) {
+                const size_t t = static_cast<size_t>(row0 + t0 + tt);
+                pre[i] = x < D ? qk[t * ldqk + g * D + x] : x < 2 * D ? qk[t * ldqk + (G + g) * D + x - D] : decay[t * ldd + h * D + x - 2 * D];
+            }
+        }
+#pragma unroll
+        for (int tt = 0; tt < TB; ++tt) pre_v[tt] = t0 + tt < n ? v[static_cast<size_t>(row0 + t0 + tt) * ldv + static_cast<size_t>(h) * V + jj] : 0.f;
+        if (BETA && lane < TB && t0 + lane < n) pre_b = beta[static_cast<size_t>(row0 + t0 + lane) * ld_beta + h];
+    };
+    fetch(0);
+    const int n_blocks = (n + TB - 1) / TB;
+    for (int block = 0; block < n_blocks; ++block) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) rows_s[lane + CELEG_WAVE * i] = pre[i];
+        if (BETA && lane < TB) beta_s[lane] = pre_b;
+        float vals[TB];
+#pragma unroll
+        for (int tt = 0; tt < TB; ++tt) vals[tt] = pre_v[tt];
+        __syncthreads();
+        if (block + 1 < n_blocks) fetch(block + 1);
+        const int count = min(TB, n - block * TB);
+        auto token = [&](int tt, float value) __attribute__((always_inline)) {
+            const float* row = rows_s + tt * ROW + sub * DPL;
+            f4 q4[NC], k4[NC], a4[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                q4[c] = *reinterpret_cast<const f4*>(row + 4 * c);
+                k4[c] = *reinterpret_cast<const f4*>(row + D + 4 * c);
+                a4[c] = *reinterpret_cast<const f4*>(row + 2 * D + 4 * c);
+            }
+            float u = value;
+            if (BETA) {
+                float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < NC; ++c)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        S[4 * c + e] *= a4[c][e];
+                        part[e] = fmaf(k4[c][e], S[4 * c + e], part[e]);
+                    }
+                u = beta_s[tt] * (value - lanes_sum<DL>((part[0] + part[1]) + (part[2] + part[3])));
+            } else {
+#pragma unroll
+                for (int c = 0; c < NC; ++c)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) S[4 * c + e] *= a4[c][e];
+            }
+            float opart[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    S[4 * c + e] = fmaf(k4[c][e], u, S[4 * c + e]);
+                    opart[e] = fmaf(q4[c][e], S[4 * c + e], opart[e]);
+                }
+            const float o = lanes_sum<DL>((opart[0] + opart[1]) + (opart[2] + opart[3]));
+            if (live && sub == 0) out[static_cast<size_t>(row0 + block * TB + tt) * ldv + static_cast<size_t>(h) * V + j] = o;
+        };
+        if (count == TB) {
+#pragma unroll
+            for (int tt = 0; tt < TB; ++tt) token(tt, vals[tt]);
+        } else {
+#pragma unroll
+            for (int tt = 0; tt < TB; ++tt)
+                if (tt < count) token(tt, vals[tt]);
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) mine[static_cast<size_t>(sub * DPL + i) * V + j] = S[i];
+    }
+}
+
 }  // namespace
 
 extern "C" int celeg_lru_gates(const void* x, int ldx, int dtype, const float* conv_w, const float* conv_b, const float* ra_t,
@@ -288,9 +397,32 @@ extern "C" int celeg_gla_prepare(const void* q, int ldq, const void* k, int ldk,
 
 extern "C" int celeg_channel_scan(const float* qk, const float* v, const float* decay, const float* beta, int ld_beta, float* state,
                                   size_t state_stride, const int* cu_seqlens, const int* seq_slot, float* out, int n_seqs, int G,
-                                  int H, int D, int V, hipStream_t stream) {
+                                  int H, int D, int V, int general, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     if (G <= 0 || H % G || D <= 0 || D > 256 || V <= 0) return static_cast<int>(hipErrorInvalidValue);
+#define CELEG_CHANNEL_BLOCKS(DL_, DPL_)                                                                                           \
+    {                                                                                                                             \
+        const int cpw = CELEG_WAVE / DL_;                                                                                         \
+        dim3 grid(n_seqs, H, (V + cpw - 1) / cpw), block(CELEG_WAVE);                                                             \
+        if (beta)                                                                                                                 \
+            hipLaunchKernelGGL((channel_scan_block_kernel<DL_, DPL_, true>), grid, block, 0, stream, qk, v, decay, beta, ld_beta, \
+                               state, state_stride, cu_seqlens, seq_slot, out, G, H, V);                                          \
+        else                                                                                                                      \
+            hipLaunchKernelGGL((channel_scan_block_kernel<DL_, DPL_, false>), grid, block, 0, stream, qk, v, decay, beta, ld_beta, \
+                               state, state_stride, cu_seqlens, seq_slot, out, G, H, V);                                          \
+        return CELEG_LAUNCH_RESULT();                                                                                             \
+    }
+    // dims that are DL lanes of a multiple of four values each; any other dim, and `general`, take the kernel below
+    if (!general) {
+        if (D == 16) CELEG_CHANNEL_BLOCKS(4, 4)
+        if (D == 32) CELEG_CHANNEL_BLOCKS(8, 4)
+        if (D == 48) CELEG_CHANNEL_BLOCKS(4, 12)
+        if (D == 64) CELEG_CHANNEL_BLOCKS(16, 4)
+        if (D == 96) CELEG_CHANNEL_BLOCKS(8, 12)
+        if (D == 128) CELEG_CHANNEL_BLOCKS(16, 8)
+        if (D == 256) CELEG_CHANNEL_BLOCKS(16, 16)
+    }
+#undef CELEG_CHANNEL_BLOCKS
 #define CELEG_CHANNEL_SCAN(P_, DPL_)                                                                                              \
     {                                                                                                                             \
         const int cpw = CELEG_WAVE / P_;                                                                                          \

@@ -66,8 +66,9 @@ def query_factor(position, q_temp):
 
 
 def distance_bias_attention(h, m, t, p):
-    """Grouped-query softmax attention over every earlier key; score(i, j) = q_i.k_j * scale * f(i)
-    - r1 ln(1 + r2 (i - j)); the heads side by side times sigmoid(W_g h), then W_o."""
+    """Grouped-query softmax attention over every earlier key (the last m["window"] keys where the
+    mixer names one); score(i, j) = q_i.k_j * scale * f(i) - r1 ln(1 + r2 (i - j)) (no bias without
+    r1); the heads side by side times sigmoid(W_g h) where there is a W_g, then W_o."""
     T = h.shape[0]
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = (h @ t[p + "q"].T).view(T, H, D)
@@ -76,16 +77,19 @@ def distance_bias_attention(h, m, t, p):
     out = torch.zeros(T, H, V, dtype=F64)
     for head in range(H):
         g = head // (H // G)
-        r1, r2 = float(t[p + "r1"][head]), float(t[p + "r2"][head])
+        r1, r2 = (float(t[p + "r1"][head]), float(t[p + "r2"][head])) if p + "r1" in t else (0.0, 0.0)
         for i in range(T):
             qi = q[i, head] * query_factor(i, m.get("q_temp"))
-            scores = torch.empty(i + 1, dtype=F64)
-            for j in range(i + 1):
-                scores[j] = float(qi @ k[j, g]) * m["scale"] - r1 * math.log(1.0 + r2 * (i - j))
+            distance = torch.arange(i, -1, -1, dtype=F64)          # i - j for j = 0 .. i
+            scores = (k[: i + 1, g] @ qi) * m["scale"] - r1 * torch.log(1.0 + r2 * distance)
+            if m.get("window"):
+                scores[distance >= m["window"]] = -math.inf
             w = torch.softmax(scores, 0)
             out[i, head] = w @ v[: i + 1, g]
-    gated = out.reshape(T, H * V) * torch.sigmoid(h @ t[p + "g"].T)
-    return gated @ t[p + "o"].T
+    out = out.reshape(T, H * V)
+    if p + "g" in t:
+        out = out * torch.sigmoid(h @ t[p + "g"].T)
+    return out @ t[p + "o"].T
 
 
 # ------------------------------------------------------------------ the pair's right side

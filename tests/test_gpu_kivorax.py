@@ -1,0 +1,647 @@
+"""The Kivorax design in the engine against the plain implementation (``plain_kivorax.py``):
+each mechanism alone through the step function (softmax attention with a distance bias and a
+factor on the query, the gated linear recurrent unit, the normed pair of the two, the delta
+rule with a decay per key channel, gated linear attention, the dense and the routed
+feed-forward, the gated row of a token table, the mixture over depth), whole models of
+several shapes in every way of cutting and batching, inputs made so that a far key, a lost
+state or a window that is one key off shows, long decoding, pages and slots used again, and
+greedy generation through the engine's entry point and scheduler.  Sizes differ from model
+to model in every number and include values that make mechanisms degenerate: one query head
+per key head and all query heads on one, a factor that changes at every position and none,
+one part of the recurrent unit and several, convolutions of one tap, one expert a token and
+all of them, a layer without feed-forward, no token table, no constant on the embedding,
+widths that are no multiple of 16, value columns that do not fill a wavefront.
+"""
+import json
+import math
+import os
+
+import pytest
+import torch
+
+import plain_kivorax as plain
+from helpers import (EngineDriver, assert_close_f32, mixed_schedule, peak_tokens, portions_schedule, random_tokens,
+                     tail_decode_schedule, whole_schedule)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+STD = 0.08
+
+
+def assert_close(got, ref, dtype, what=""):
+    """32-bit: the shared bound (1e-4 of the largest logit).  bfloat16: relative RMS error <= 6e-2, and
+    every row's max |d| <= 1e-1 * max |ref| but for one row in fifty (at least one).  The pair norms
+    both mixers' rounded outputs and the token input norms its own, so rounding alone moves these
+    narrow models' logits by one to three percent relative RMS, the same however a prompt is cut.
+    Single rows move more where the design itself hangs on a close call that rounding decides: the
+    first token's read-out of a matrix state is (q.k) v, whose norm over the values keeps only the
+    sign of q.k, and a router that takes one expert changes the expert when two scores are close.
+    Such rows are the same in every schedule; the faults these tests look for move many rows by tens
+    of percent, and the 32-bit runs of the same schedules hold every row to 1e-4."""
+    if dtype in ("float32", torch.float32):
+        return assert_close_f32(got, ref, what)
+    got, ref = torch.as_tensor(got).double(), torch.as_tensor(ref).double()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite logits"
+    d = got - ref
+    rel = float(d.pow(2).mean().sqrt() / ref.pow(2).mean().sqrt())
+    rows = d.abs().reshape(-1, d.shape[-1]).max(-1).values / ref.abs().max()
+    over = int((rows > 1e-1).sum())
+    assert rel <= 6e-2 and over <= max(1, rows.numel() // 50), \
+        f"{what}: rel rms {rel:.3e} (<= 6e-2), {over} of {rows.numel()} rows over 1e-1 of the largest logit, worst {float(rows.max()):.3e}"
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts, top, ff):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def pair(heads, kv_heads, dim, vdim, scale, q_temp, inner, blocks, taps, mlp):
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if q_temp:
+        left["q_temp"] = {"coef": q_temp[0], "every": q_temp[1]}
+    return {"type": "parallel", "mixer": {"left": left, "right": {"width": inner, "blocks": blocks, "conv": taps}}, "mlp": mlp}
+
+
+def channel_delta(heads, kv_heads, dim, vdim, taps, mlp, decay_rank=6, gate_rank=5):
+    return {"type": "channel_delta", "mlp": mlp,
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": taps, "decay_rank": decay_rank, "gate_rank": gate_rank}}
+
+
+def gla(heads, dim, vdim, tau, mlp, decay_rank=7):
+    return {"type": "gla", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau, "decay_rank": decay_rank}, "mlp": mlp}
+
+
+# heads of sizes the matrix cores take (keys and values of different sizes), a factor that changes every 16 positions
+V1 = {"architecture": "Kivorax", "vocab": 310, "width": 96, "norm": {"eps": 1e-5}, "embedding": {"scale": 2.0}, "token_side": {"dim": 12},
+      "layers": [pair(4, 2, 32, 64, 0.2, (0.25, 16), 48, 3, 3, dense(80)), channel_delta(4, 2, 16, 24, 4, moe(6, 2, 32)),
+                 gla(3, 32, 40, 8.0, None), pair(3, 3, 64, 32, 0.15, None, 40, 1, 2, moe(6, 2, 32))]}
+# no constant on the embedding, no token table, a width that is no multiple of 16, one tap, all query heads on
+# one key head, a factor that changes at every position, every expert chosen, heads no kernel in registers takes
+V2 = {"architecture": "Kivorax", "vocab": 211, "width": 72, "norm": {"eps": 3e-6},
+      "layers": [gla(2, 12, 20, 3.0, dense(40)), pair(5, 1, 8, 20, 0.35, (0.1, 1), 36, 4, 1, None),
+                 channel_delta(3, 1, 40, 12, 5, moe(3, 3, 24)), channel_delta(2, 2, 8, 70, 1, dense(40), decay_rank=2, gate_rank=11)]}
+# heads of 128 and 96, one expert a token, the pair last and first, states of 64 x 64 and 64 x 32
+V3 = {"architecture": "Kivorax", "vocab": 260, "width": 128, "norm": {"eps": 1e-4}, "embedding": {"scale": 0.5}, "token_side": {"dim": 8},
+      "layers": [pair(2, 2, 128, 96, 0.09, (0.4, 50), 128, 2, 4, moe(4, 1, 48)), gla(2, 64, 64, 16.0, moe(4, 1, 48)),
+                 channel_delta(8, 2, 64, 32, 3, dense(64)), pair(4, 1, 96, 128, 0.1, (0.2, 64), 24, 2, 3, dense(64))]}
+MODELS = {"V1": (V1, 31), "V2": (V2, 32), "V3": (V3, 33)}
+LENGTHS = {"V1": [40, 57, 90, 128, 65, 33], "V2": [45, 130, 64, 100, 17, 33], "V3": [31, 32, 150, 64, 49, 80]}
+SCHEDULES = {"whole": whole_schedule, "tail12": lambda reqs: tail_decode_schedule(reqs, tail=12),
+             "portions": portions_schedule, "mixed": mixed_schedule}
+
+
+def write_model(folder, cfg, seed, storage=torch.float32, std=STD, replace=None, change=None):
+    """A model folder of random tensors for ``cfg``; ``replace``: name -> tensor, ``change``:
+    name -> function of the drawn tensor."""
+    from celeg_amd import native
+    from celeg_amd.weights import random_tensors
+    from celeg_amd.weights.safetensors_io import write_safetensors
+    expected = native.describe_config(cfg)["expected_tensors"]
+    tensors = random_tensors(expected, seed, std, torch.float32)
+    for name, t in (replace or {}).items():
+        assert tensors[name].shape == t.shape, name
+        tensors[name] = t.float()
+    for name, fn in (change or {}).items():
+        tensors[name] = fn(tensors[name])
+    tensors = {k: v.to(storage).contiguous() for k, v in tensors.items()}
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as fh:
+        json.dump(cfg, fh)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    return str(folder)
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    made = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in made:
+            cfg, seed = MODELS[name]
+            storage = torch.float32 if dtype == "float32" else torch.bfloat16
+            made[(name, dtype)] = write_model(tmp_path_factory.mktemp(f"{name}_{dtype}"), cfg, seed, storage)
+        return made[(name, dtype)]
+    return get
+
+
+_plain = {}
+
+
+def requests_of(name):
+    cfg, seed = MODELS[name]
+    return {f"r{i}": random_tokens(cfg["vocab"], n, seed=100 * seed + i) for i, n in enumerate(LENGTHS[name])}
+
+
+def plain_logits(folder, key, requests):
+    if key not in _plain:
+        cfg, W = plain.load_model_folder(folder)
+        _plain[key] = {rid: plain.forward(cfg, W, toks) for rid, toks in requests.items()}
+    return _plain[key]
+
+
+def load(folder, dtype, steps, max_requests=4, **kw):
+    from celeg_amd.engine import load_model
+    max_tokens = peak_tokens(steps)
+    lm = load_model(folder, dtype=dtype, device=DEV, page_tokens=16, n_pages=max_tokens // 16, max_requests=max_requests,
+                    max_context=max_tokens, max_batched_tokens=max(max_tokens, 64), **kw)
+    return lm, max_tokens
+
+
+@pytest.mark.parametrize("mode", list(SCHEDULES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(MODELS))
+def test_engine_matches_plain(folders, name, dtype, mode):
+    """Whole prompts; prefill then 12 tokens one by one; portions down to two tokens (and single
+    ones) that cross page borders; four live requests with pages and slots used again."""
+    folder = folders(name, dtype)
+    reqs = requests_of(name)
+    steps = SCHEDULES[mode](reqs)
+    lm, max_tokens = load(folder, dtype, steps)
+    got = EngineDriver(lm).run(steps)
+    ref = plain_logits(folder, (name, dtype), reqs)
+    for rid in reqs:
+        assert_close(got[rid], ref[rid], dtype, f"{name}/{dtype}/{mode}/{rid}")
+    lm.cache.check()
+    assert lm.cache.n_free_slots == 4 and lm.cache.free_pages() == [max_tokens // 16] * len(lm.cache.free_pages())
+    paths = lm.paths()
+    assert paths["attention_biased"] > 0 and paths["channel_scan"] > 0 and paths["linear_recurrent_unit"] > 0
+    if dtype == "bfloat16" and name != "V2":
+        assert paths["attention_biased_rows"] + paths["attention_biased_decode"] > 0     # the matrix cores took these heads
+
+
+@pytest.mark.parametrize("name", ["V1", "V2"])
+def test_residual_stream_after_every_layer(folders, tmp_path, monkeypatch, name):
+    """32-bit: the stream behind each layer (after the token input and the mixture over depth) as
+    CELEG_DUMP_HIDDEN writes it, for a prompt's portion and two single tokens, against the plain
+    layers: the first layer that differs is where a fault lies."""
+    import numpy as np
+    from celeg_amd.engine import StepEntry, load_model
+    cfg, _ = MODELS[name]
+    folder = folders(name, "float32")
+    _, W = plain.load_model_folder(folder)
+    toks = random_tokens(cfg["vocab"], 23, seed=2)
+    _, after = plain.forward(cfg, W, toks, return_layers=True)
+    dump = str(tmp_path / "hidden")
+    monkeypatch.setenv("CELEG_DUMP_HIDDEN", dump)
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=8, max_requests=2, max_batched_tokens=64)
+    monkeypatch.delenv("CELEG_DUMP_HIDDEN")
+    slot = lm.cache.open()
+    assert lm.cache.prepare(slot, 0, 23)
+    for k, (start, n) in enumerate([(0, 21), (21, 1), (22, 1)]):
+        lm.runner.step([StepEntry(slot, start, toks[start:start + n], [n - 1])])
+        for i in range(len(cfg["layers"])):
+            rows = np.fromfile(os.path.join(dump, f"step{k}_layer{i}.f32"), dtype="<f4").reshape(n, cfg["width"])
+            assert_close_f32(torch.from_numpy(rows), after[i][start:start + n], f"step {k}, layer {i}")
+    lm.close()
+
+
+def test_batches_of_unequal_requests_equal_each_alone(folders):
+    """In 32-bit a row's logits do not depend on what else is in the batch or on how the prompt was
+    cut, beyond the rounding of 32-bit sums taken in another order: held to 2e-5 of the largest logit."""
+    folder = folders("V1", "float32")
+    reqs = requests_of("V1")
+    alone_steps, mixed_steps = whole_schedule(reqs), mixed_schedule(reqs, seed=3)
+    lm, _ = load(folder, "float32", alone_steps)
+    alone = EngineDriver(lm).run(alone_steps)
+    lm2, _ = load(folder, "float32", mixed_steps)
+    mixed = EngineDriver(lm2).run(mixed_steps)
+    for rid in reqs:
+        assert float((alone[rid] - mixed[rid]).abs().max()) <= 2e-5 * float(alone[rid].abs().max()), rid
+
+
+# ------------------------------------------------------------------ inputs made so that a fault shows
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_state_that_remembers_hundreds_of_tokens(tmp_path, dtype):
+    """Decays close to one in all three kinds of state: what the first tokens wrote still shows 300
+    tokens later (the plain model run on the last 150 tokens alone gives other logits), so a state
+    that is lost, zeroed or taken from another slot between steps cannot pass."""
+    cfg = {"architecture": "Kivorax", "vocab": 140, "width": 64, "norm": {"eps": 1e-5},
+           "layers": [channel_delta(4, 2, 16, 20, 3, dense(32)), gla(2, 24, 16, 64.0, None),
+                      pair(2, 1, 32, 32, 0.2, None, 32, 2, 3, None)]}
+    slow = {"l0.mix.A_log": torch.full((4,), -7.0), "l1.mix.a2.b": torch.full((48,), 3.0), "l2.mix.right.lam": torch.full((32,), -9.0)}
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = write_model(tmp_path / "far", cfg, 7, storage, std=0.1, replace=slow)
+    c, W = plain.load_model_folder(folder)
+    toks = random_tokens(cfg["vocab"], 300, seed=3)
+    ref = plain.forward(c, W, toks)
+    # every layer by itself remembers: without its slow decay the last logits are others
+    tail_alone = plain.forward(c, W, toks[150:])
+    assert float((ref[-1] - tail_alone[-1]).abs().max()) > 0.02 * float(ref[-1].abs().max())
+    reqs = {"far": toks, "other": random_tokens(cfg["vocab"], 90, seed=4)}
+    ref = {"far": ref, "other": plain.forward(c, W, reqs["other"])}
+    for steps in (tail_decode_schedule(reqs, tail=40), portions_schedule(reqs, sizes=(97, 2, 130, 31, 16, 1, 64, 3)),
+                  mixed_schedule(reqs, seed=5, decode_tail=10)):
+        lm, _ = load(folder, dtype, steps)
+        got = EngineDriver(lm).run(steps)
+        for rid in reqs:
+            assert_close(got[rid], ref[rid], dtype, f"far state/{dtype}/{rid}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_over_many_pages(folders, dtype):
+    """A short prompt, then 200 tokens one by one (steps replayed from a recorded graph), over a
+    dozen page borders and four changes of the query's factor."""
+    folder = folders("V3", dtype)
+    toks = random_tokens(V3["vocab"], 215, seed=77)
+    steps = tail_decode_schedule({"long": toks}, tail=200)
+    lm, _ = load(folder, dtype, steps)
+    got = EngineDriver(lm).run(steps)["long"]
+    c, W = plain.load_model_folder(folder)
+    assert_close(got, plain.forward(c, W, toks), dtype, "long decoding")
+    assert lm.runner.counters()["graph_replays"] > 100
+
+
+def test_pages_and_slots_used_again(folders):
+    """Ten requests through two slots and a pool of six pages: every page and state slot serves
+    several requests, and each request's logits equal the plain ones (a state that is not zeroed
+    when its slot is given out again would show at the request's first token)."""
+    folder = folders("V1", "float32")
+    reqs = {f"q{i}": random_tokens(V1["vocab"], n, seed=500 + i) for i, n in enumerate([30, 18, 33, 16, 5, 47, 31, 2, 40, 17])}
+    steps = mixed_schedule(reqs, max_live=2, seed=4, decode_tail=6)
+    from celeg_amd.engine import load_model
+    lm = load_model(folder, dtype="float32", device=DEV, page_tokens=16, n_pages=6, max_requests=2, max_context=64,
+                    max_batched_tokens=128)
+    got = EngineDriver(lm).run(steps)
+    c, W = plain.load_model_folder(folder)
+    for rid, toks in reqs.items():
+        assert_close_f32(got[rid], plain.forward(c, W, toks), rid)
+    assert all(n == 6 for n in lm.cache.free_pages())
+
+
+# ------------------------------------------------------------------ generation through the entry point
+@pytest.mark.parametrize("name", ["V1", "V2"])
+def test_greedy_generation_through_the_entry_point(folders, name):
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GenerationConfig
+    folder = folders(name, "float32")
+    cfg, W = plain.load_model_folder(folder)
+    prompts = [random_tokens(cfg["vocab"], n, seed=40 + n) for n in (5, 23, 1, 37, 12)]
+    engine = Engine.from_folder(folder, dtype="float32", device=DEV, max_active_requests=3, max_batched_tokens=64,
+                                prefill_chunk_tokens=16, context=128, n_pages=24)
+    greedy = GenerationConfig(temperature=0.0, repetition_penalty=1.0)
+    outs = engine.generate(prompts, max_new_tokens=20, generation=greedy, eos_token_ids=[])
+    for prompt, out in zip(prompts, outs):
+        assert out == plain.greedy(cfg, W, prompt, 20)
+    engine.close()
+
+
+def test_command_line(folders, tmp_path):
+    """``bin/celeg-run`` on a model folder of the design: greedy tokens and the prompt's last logits."""
+    import subprocess
+    import sys
+    import numpy as np
+    folder = folders("V2", "float32")
+    cfg, W = plain.load_model_folder(folder)
+    prompt = random_tokens(cfg["vocab"], 19, seed=5)
+    dump = str(tmp_path / "logits.f32")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "celeg-run"), "--model", folder, "--dtype", "float32", "--prompt",
+                           ",".join(map(str, prompt)), "--max-new-tokens", "8", "--repetition-penalty", "1.0", "--context", "128",
+                           "--runtime-tokens", "--dump-logits", dump], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr
+    line = [l for l in proc.stdout.splitlines() if l.startswith("CELEG_GENERATED_TOKEN_IDS=")][0]
+    assert json.loads(line.split("=", 1)[1]) == plain.greedy(cfg, W, prompt, 8)
+    logits = np.fromfile(dump, dtype="<f4")
+    assert_close_f32(torch.from_numpy(logits.copy()), plain.forward(cfg, W, prompt)[-1], "command line")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_program(folders, tmp_path, dtype):
+    """``bin/trace_run`` in a process of its own: four schedules one after the other, a pool sized for
+    the live requests only, logits read from the files it writes."""
+    from helpers import TraceClient
+    folder = folders("V1", dtype)
+    reqs = requests_of("V1")
+    ref = plain_logits(folder, ("V1", dtype), reqs)
+    all_steps = []
+    for tag, make in (("w", whole_schedule), ("t", tail_decode_schedule), ("p", portions_schedule), ("m", mixed_schedule)):
+        for s in make({f"{tag}{rid}": toks for rid, toks in reqs.items()}):
+            all_steps.append(dict(s, step=len(all_steps)))
+    client = TraceClient(folder, dtype, str(tmp_path), peak_tokens(all_steps))
+    got = {}
+    for s in all_steps:
+        logits = client.step(s["step"], s["entries"], s["end"])
+        row = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got.setdefault(e["id"], []).append(torch.as_tensor(logits[row]))
+                row += 1
+    assert client.close() == 0
+    for rid_tagged, rows in got.items():
+        assert_close(torch.stack(rows), ref[rid_tagged[1:]], dtype, f"trace/{dtype}/{rid_tagged}")
+
+
+# ------------------------------------------------------------------ each mechanism alone
+def alone_architecture():
+    """"KivoraxPartsAlone": one block put together from what the configuration spells out, both
+    sub-layers reading the stream as it is; the embedding table is the input x (tokens 0..T-1), the
+    head gives the stream's rows back."""
+    from celeg_amd.config import LayerSpec, ModelSpec, PartSpec, RunStep, register_architecture, registered_architectures
+    if "KivoraxPartsAlone" in registered_architectures():
+        return
+
+    def build(cfg, shapes):
+        W, rows = cfg["width"], cfg["rows"]
+        part = lambda key, neutral: PartSpec.from_json(cfg[key]) if cfg.get(key) else neutral
+        maybe = lambda key: PartSpec.from_json(cfg[key]) if cfg.get(key) else None
+        block = LayerSpec(part("mixer", PartSpec("none", {"width": W})), PartSpec("identity"), part("ffn", PartSpec("none")),
+                          PartSpec("identity"), "parallel", token_input=maybe("token_input"), depth_mix=maybe("depth_mix"))
+        return ModelSpec("KivoraxPartsAlone", rows, W, 512, PartSpec("embedding", {"vocab": rows, "width": W}, {"table": "x"}),
+                         (block,), (RunStep(0, None, False),), PartSpec("identity"), PartSpec("hidden", {"width": W}))
+    register_architecture("KivoraxPartsAlone", build)
+
+
+CUT = (5, 2, 9, 1, 3, 17)
+
+
+def run_alone(tmp_path, cfg, tensors, cut=CUT, dtype="float32", knobs=None, n_pages=8):
+    """What the block makes of rows 0..T-1, in portions."""
+    from celeg_amd.engine import load_model
+    from celeg_amd.weights.safetensors_io import write_safetensors
+    alone_architecture()
+    cfg = dict(cfg, architectures=["KivoraxPartsAlone"])
+    os.makedirs(tmp_path, exist_ok=True)
+    with open(os.path.join(tmp_path, "config.json"), "w") as fh:
+        json.dump(cfg, fh)
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    write_safetensors(os.path.join(tmp_path, "model.safetensors"), {k: v.to(storage).contiguous() for k, v in tensors.items()})
+    steps = portions_schedule({"x": list(range(cfg["rows"]))}, sizes=cut)
+    lm = load_model(str(tmp_path), dtype=dtype, device=DEV, page_tokens=16, n_pages=n_pages, max_requests=2, max_context=16 * n_pages,
+                    max_batched_tokens=max(64, max(cut)))
+    for k, v in (knobs or {}).items():
+        lm.set_knob(k, v)
+    return EngineDriver(lm).run(steps)["x"].double(), lm
+
+
+def attention_case(T, W_, H, G, D, V, scale, q_temp=None, window=None, bias=True, gate=True, seed=1, x_std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)
+    t = {"x": r(T, W_) * x_std, "q": r(H * D, W_) * 0.3, "k": r(G * D, W_) * 0.3, "v": r(G * V, W_) * 0.3, "o": r(W_, H * V) * 0.3}
+    if bias:
+        t["r1"], t["r2"] = 0.5 + torch.rand(H, generator=g), 0.2 + torch.rand(H, generator=g)
+    if gate:
+        t["g"] = r(H * V, W_) * 0.3
+    params = {"width": W_, "heads": H, "kv_heads": G, "head_dim": D, "v_dim": V, "scale": scale, "distance_bias": bias,
+              "gate": "sigmoid" if gate else "none"}
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": V, "scale": scale}
+    if q_temp:
+        params["query_temperature"] = {"coef": q_temp[0], "every": q_temp[1]}
+        m["q_temp"] = {"coef": q_temp[0], "every": q_temp[1]}
+    if window:
+        params["window"] = m["window"] = window
+    part = {"kind": "biased_attention", "params": params, "tensors": {k: k for k in t if k != "x"}}
+    return t, m, part
+
+
+@pytest.mark.parametrize("q_temp,window,bias,gate", [((0.3, 7), None, True, True), (None, None, True, False), ((0.5, 1), 16, False, True),
+                                                     ((0.2, 100), 17, True, True), (None, 1, True, True)])
+def test_distance_bias_attention_alone(tmp_path, q_temp, window, bias, gate):
+    T, W_ = 45, 40
+    t, m, part = attention_case(T, W_, 6, 3, 12, 20, 0.3, q_temp, window, bias, gate)
+    got, _ = run_alone(tmp_path, {"width": W_, "rows": T, "mixer": part}, t)
+    Wd = {k: v.double() for k, v in t.items()}
+    assert_close_f32(got, Wd["x"] + plain.distance_bias_attention(Wd["x"], m, Wd, ""), "attention with a distance bias alone")
+
+
+def test_the_distance_bias_and_the_factor_show():
+    """The plain attention without the bias, with the two numbers swapped, with the factor one
+    position late or with a window one key off differs by far more than any tolerance."""
+    t, m, _ = attention_case(60, 24, 2, 1, 16, 16, 0.5, (0.5, 4), None)
+    t["r1"], t["r2"] = torch.tensor([1.5, 0.4]), torch.tensor([0.3, 2.0])
+    Wd = {k: v.double() for k, v in t.items()}
+
+    def moved(mixer, tensors, by):
+        right = plain.distance_bias_attention(Wd["x"], by, Wd, "")
+        return float((plain.distance_bias_attention(Wd["x"], mixer, tensors, "") - right).abs().max()) / float(right.abs().max())
+    assert moved(m, {k: v for k, v in Wd.items() if k not in ("r1", "r2")}, m) > 0.1
+    assert moved(m, dict(Wd, r1=Wd["r2"], r2=Wd["r1"]), m) > 0.1
+    assert moved(dict(m, q_temp=None), Wd, m) > 0.1
+    assert moved(dict(m, q_temp={"coef": 0.5, "every": 5}), Wd, m) > 0.01       # the factor's steps one position late in five
+    for other in (8, 10):
+        assert moved(dict(m, window=other), Wd, dict(m, window=9)) > 0.1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_key_far_back_among_hundreds(tmp_path, dtype):
+    """Row 3's long key and the queries of rows 250 (inside a prompt's portion) and 299 (decoded alone)
+    point the same way, so those rows' weight sits on a key 247 and 296 positions back,
+    across a dozen and a half pages and the distance bias; left out, the rows' outputs are others."""
+    T, W_, H, D = 300, 32, 2, 32
+    t, m, part = attention_case(T, W_, H, H, D, D, 0.25, (0.3, 128), None, True, True, seed=5, x_std=0.3)
+    t["k"] = t["q"].clone()                      # a row's own direction scores high against itself
+    t["r1"] = torch.tensor([0.3, 0.6])
+    direction = torch.randn(W_, generator=torch.Generator().manual_seed(9))
+    direction = direction / direction.norm()
+    for row, length in ((3, 8.0), (250, 2.0), (299, 2.0)):      # (a row's own key scores a quarter of row 3's)
+        t["x"][row] = length * direction
+    Wd = {k: v.double() for k, v in t.items()}
+    want = Wd["x"] + plain.distance_bias_attention(Wd["x"], m, Wd, "")
+    without = Wd["x"].clone()
+    without[3] = Wd["x"][4]
+    lost = Wd["x"] + plain.distance_bias_attention(without, m, Wd, "")
+    for row in (250, 299):
+        assert float((want[row] - lost[row]).abs().max()) > 0.1 * float(want[row].abs().max())
+    got, lm = run_alone(tmp_path, {"width": W_, "rows": T, "mixer": part}, t, cut=(130, 2, 97, 31, 16, 1, 7, 3, 2, 1, 1, 1, 1, 1, 1, 1, 1, 1),
+                        dtype=dtype, n_pages=20)
+    if dtype == "float32":
+        assert_close_f32(got, want, "a far key")
+    else:
+        ref = (Wd["x"].bfloat16().double() + plain.distance_bias_attention(
+            Wd["x"].bfloat16().double(), m, {k: v.bfloat16().double() for k, v in Wd.items()}, ""))
+        for row in (250, 299, 120):
+            assert float((got[row] - ref[row]).abs().max()) <= 0.03 * float(ref[row].abs().max()), row
+        assert lm.paths()["attention_biased_rows"] > 0 and lm.paths()["attention_biased_decode"] > 0
+
+
+@pytest.mark.parametrize("D,V", [(32, 32), (64, 128), (96, 64), (128, 96), (32, 128)])
+def test_matrix_core_attention_equals_the_general_kernel(tmp_path, D, V):
+    """bfloat16: the kernels on the matrix cores against the kernel that scores key by key, on the
+    same pages, with windows that end before, at and behind the borders of pages and of the blocks
+    of 64 keys and with none, in whole prompts, portions and single tokens.  The two differ in the
+    rounding of the weights to bfloat16 only."""
+    T, W_ = 300, 64
+    for window in (None, 7, 64, 65):
+        t, m, part = attention_case(T, W_, 4, 2, D, V, D ** -0.5, (0.3, 32), window, True, True, seed=D + V, x_std=1.5)
+        got = {}
+        for form, cut in (("general", (15, 2, 17, 1, 130, 3, 16, 64)), (-1, (15, 2, 17, 1, 130, 3, 16, 64)), (0, (15, 2, 17, 1, 130, 3, 16, 64)),
+                          (1, (15, 2, 17, 1, 130, 3, 16, 64)), (-1, (300,)), (-1, (270,) + (1,) * 30)):
+            knobs = {"use_biased_mfma": 0} if form == "general" else {"biased_rows_form": form}
+            out, lm = run_alone(tmp_path / f"{window}_{form}_{len(cut)}", {"width": W_, "rows": T, "mixer": part}, t, cut=cut, dtype="bfloat16",
+                                knobs=knobs, n_pages=20)
+            took = lm.paths()["attention_biased_rows"] + lm.paths()["attention_biased_decode"]
+            assert (took > 0) == (form != "general")
+            got[(form, len(cut))] = out
+        ref = got[("general", 8)]
+        for key, out in got.items():
+            rel = float((out - ref).pow(2).mean().sqrt() / ref.pow(2).mean().sqrt())
+            assert rel <= 1e-2, f"heads of {D} and {V}, window {window}, form {key}: rel rms {rel:.3e}"
+
+
+def lru_case(T, W_, C, B, taps, seed=2):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)
+    n = C // B
+    t = {"x_in": r(T, W_), "y": r(C, W_) * 0.3, "y.b": r(C) * 0.3, "x": r(C, W_) * 0.3, "x.b": r(C) * 0.3, "conv": r(C, taps) * 0.5,
+         "conv.b": r(C) * 0.3, "ra": r(B, n, n) * 0.4, "ra.b": r(B, n) * 0.5, "ri": r(B, n, n) * 0.4, "ri.b": r(B, n) * 0.5,
+         "lam": r(C) - 2.0, "o": r(W_, C) * 0.3}
+    names = {"y": "y", "y_bias": "y.b", "x": "x", "x_bias": "x.b", "conv": "conv", "conv_bias": "conv.b", "ra": "ra", "ra_bias": "ra.b",
+             "ri": "ri", "ri_bias": "ri.b", "lam": "lam", "o": "o"}
+    part = {"kind": "linear_recurrent_unit", "params": {"width": W_, "inner": C, "blocks": B, "taps": taps, "decay_scale": 8.0}, "tensors": names}
+    return t, {"width": C, "blocks": B, "conv": taps}, part
+
+
+@pytest.mark.parametrize("C,B,taps", [(36, 3, 4), (40, 1, 1), (70, 5, 2), (256, 2, 4), (12, 12, 3)])
+def test_linear_recurrent_unit_alone(tmp_path, C, B, taps):
+    T, W_ = 45, 40
+    t, m, part = lru_case(T, W_, C, B, taps)
+    tensors = {("table" if k == "x_in" else k): v for k, v in t.items()}
+    part = dict(part, tensors=dict(part["tensors"]))
+    got, lm = run_alone_named(tmp_path, W_, T, part, tensors)
+    Wd = {k: v.double() for k, v in t.items()}
+    assert_close_f32(got, Wd["x_in"] + plain.gated_linear_recurrent_unit(Wd["x_in"], m, Wd, ""), "linear recurrent unit alone")
+    assert lm.paths()["linear_recurrent_unit"] > 0
+
+
+def run_alone_named(tmp_path, W_, T, part, tensors, **kw):
+    """As ``run_alone`` for parts one of whose tensors is called "x" itself: the input is the tensor "table"."""
+    from celeg_amd.config import LayerSpec, ModelSpec, PartSpec, RunStep, register_architecture, registered_architectures
+    if "KivoraxPartsAloneTable" not in registered_architectures():
+        def build(cfg, shapes):
+            W, rows = cfg["width"], cfg["rows"]
+            block = LayerSpec(PartSpec.from_json(cfg["mixer"]), PartSpec("identity"), PartSpec("none"), PartSpec("identity"), "parallel")
+            return ModelSpec("KivoraxPartsAloneTable", rows, W, 512, PartSpec("embedding", {"vocab": rows, "width": W}, {"table": "table"}),
+                             (block,), (RunStep(0, None, False),), PartSpec("identity"), PartSpec("hidden", {"width": W}))
+        register_architecture("KivoraxPartsAloneTable", build)
+    from celeg_amd.engine import load_model
+    from celeg_amd.weights.safetensors_io import write_safetensors
+    os.makedirs(tmp_path, exist_ok=True)
+    with open(os.path.join(tmp_path, "config.json"), "w") as fh:
+        json.dump({"architectures": ["KivoraxPartsAloneTable"], "width": W_, "rows": T, "mixer": part}, fh)
+    write_safetensors(os.path.join(tmp_path, "model.safetensors"), {k: v.float().contiguous() for k, v in tensors.items()})
+    steps = portions_schedule({"x": list(range(T))}, sizes=CUT)
+    lm = load_model(str(tmp_path), dtype="float32", device=DEV, page_tokens=16, n_pages=8, max_requests=2, max_context=128,
+                    max_batched_tokens=64)
+    return EngineDriver(lm).run(steps)["x"].double(), lm
+
+
+def test_normed_pair_alone(tmp_path):
+    """The mean of the two mixers' outputs, each normed over the width with a weight of its own."""
+    torch.manual_seed(8)
+    T, W_, eps = 45, 40, 1e-4
+    ta, ma, pa = attention_case(T, W_, 4, 2, 8, 12, 0.3, (0.3, 5))
+    tr, mr, pr = lru_case(T, W_, 24, 2, 3)
+    tensors = {"table": ta["x"], "left.out": 1 + 0.3 * torch.randn(W_), "right.out": 1 + 0.3 * torch.randn(W_)}
+    names = {"left_out": "left.out", "right_out": "right.out"}
+    for k, v in ta.items():
+        if k != "x":
+            tensors["left." + k] = v
+            names["left." + k] = "left." + k
+    for key, name in pr["tensors"].items():
+        tensors["right." + name] = tr[name]
+        names["right." + key] = "right." + name
+    inner = lambda p: {"kind": p["kind"], "params": p["params"], "tensors": {}}
+    part = {"kind": "normed_pair", "params": {"width": W_, "eps": eps, "factor": 0.5, "left": inner(pa), "right": inner(pr)}, "tensors": names}
+    got, _ = run_alone_named(tmp_path, W_, T, part, tensors)
+    Wd = {k: v.double() for k, v in tensors.items()}
+    want = Wd["table"] + plain.normed_pair(Wd["table"], {"left": ma, "right": mr}, Wd, "", eps)
+    assert_close_f32(got, want, "normed pair alone")
+
+
+# (dims of 16, 32, 48, 64, 96, 128 and 256 keep the state in registers; the others do not)
+DIMS = [(4, 2, 12, 20, 3), (3, 3, 8, 70, 1), (2, 1, 40, 8, 6), (4, 2, 16, 100, 4), (2, 2, 32, 64, 2), (2, 1, 48, 20, 3), (3, 1, 64, 48, 4),
+        (2, 2, 96, 16, 2), (2, 1, 128, 24, 2), (1, 1, 256, 70, 3)]
+
+
+@pytest.mark.parametrize("H,G,D,V,taps", DIMS)
+def test_channel_delta_rule_alone(tmp_path, H, G, D, V, taps):
+    torch.manual_seed(2)
+    T, W_, ra, rg = 45, 32, 5, 9
+    t = {"x": torch.randn(T, W_), "q": torch.randn(G * D, W_) * 0.3, "k": torch.randn(G * D, W_) * 0.3, "v": torch.randn(H * V, W_) * 0.3,
+         "q.conv": torch.randn(G * D, taps) * 0.5, "k.conv": torch.randn(G * D, taps) * 0.5, "v.conv": torch.randn(H * V, taps) * 0.5,
+         "b": torch.randn(H, W_) * 0.3, "A_log": torch.randn(H) - 1.0, "dt_bias": torch.randn(H * D), "a1": torch.randn(ra, W_) * 0.3,
+         "a2": torch.randn(H * D, ra) * 0.5, "g1": torch.randn(rg, W_) * 0.3, "g2": torch.randn(H * V, rg) * 0.5,
+         "norm": 1 + 0.2 * torch.randn(V), "o": torch.randn(W_, H * V) * 0.3}
+    names = {"q": "q", "k": "k", "v": "v", "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv", "b": "b", "A_log": "A_log",
+             "dt_bias": "dt_bias", "a1": "a1", "a2": "a2", "g1": "g1", "g2": "g2", "norm": "norm", "o": "o"}
+    params = {"width": W_, "heads": H, "kv_heads": G, "dim": D, "vdim": V, "taps": taps, "eps": 1e-4, "decay": "channel", "decay_rank": ra,
+              "gate": "sigmoid", "gate_rank": rg}
+    Wd = {k: v.double() for k, v in t.items()}
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": V, "conv": taps}
+    want = Wd["x"] + plain.channel_delta_rule(Wd["x"], m, Wd, "", 1e-4)
+    for general in (0, 1):
+        got, lm = run_alone(tmp_path / str(general), {"width": W_, "rows": T, "mixer": {"kind": "gated_delta_rule", "tensors": names, "params": params}},
+                            t, knobs={"delta_general": general})
+        assert_close_f32(got, want, f"channel delta rule alone (general {general})")
+        assert lm.paths()["channel_scan"] > 0
+
+
+@pytest.mark.parametrize("H,D,V", [(3, 12, 20), (2, 16, 100), (2, 32, 64), (2, 48, 40), (1, 64, 64), (2, 96, 8), (1, 128, 24), (1, 256, 70), (5, 8, 8)])
+@pytest.mark.parametrize("tau", [1.0, 16.0])
+def test_gated_linear_attention_alone(tmp_path, H, D, V, tau):
+    torch.manual_seed(3)
+    T, W_, ra = 45, 32, 6
+    t = {"x": torch.randn(T, W_), "q": torch.randn(H * D, W_) * 0.3, "k": torch.randn(H * D, W_) * 0.3, "v": torch.randn(H * V, W_) * 0.3,
+         "g": torch.randn(H * V, W_) * 0.3, "a1": torch.randn(ra, W_) * 0.3, "a2": torch.randn(H * D, ra) * 0.5, "a2.b": torch.randn(H * D) + 1.0,
+         "norm": 1 + 0.2 * torch.randn(V), "o": torch.randn(W_, H * V) * 0.3}
+    names = {"q": "q", "k": "k", "v": "v", "g": "g", "a1": "a1", "a2": "a2", "a2_bias": "a2.b", "norm": "norm", "o": "o"}
+    params = {"width": W_, "heads": H, "dim": D, "vdim": V, "tau": tau, "decay_rank": ra, "eps": 1e-4}
+    Wd = {k: v.double() for k, v in t.items()}
+    want = Wd["x"] + plain.gated_linear_attention(Wd["x"], {"heads": H, "dim": D, "vdim": V, "tau": tau}, Wd, "", 1e-4)
+    for general in (0, 1):
+        got, _ = run_alone(tmp_path / str(general), {"width": W_, "rows": T, "mixer": {"kind": "gated_linear_attention", "tensors": names, "params": params}},
+                           t, knobs={"delta_general": general})
+        assert_close_f32(got, want, f"gated linear attention alone (general {general})")
+
+
+def test_dense_feed_forward_alone(tmp_path):
+    torch.manual_seed(4)
+    T, W_, ff = 29, 36, 50
+    t = {"x": torch.randn(T, W_) * 2, "up": torch.randn(ff, W_) * 0.3, "up.b": torch.randn(ff), "down": torch.randn(W_, ff) * 0.3, "down.b": torch.randn(W_)}
+    part = {"kind": "mlp", "params": {"width": W_, "ff": ff, "activation": "gelu_tanh", "bias": True},
+            "tensors": {"up": "up", "up_bias": "up.b", "down": "down", "down_bias": "down.b"}}
+    got, _ = run_alone(tmp_path, {"width": W_, "rows": T, "ffn": part}, t)
+    Wd = {k: v.double() for k, v in t.items()}
+    assert_close_f32(got, Wd["x"] + plain.dense_mlp(Wd["x"], Wd, ""), "dense feed-forward alone")
+
+
+@pytest.mark.parametrize("experts,top", [(5, 2), (4, 1), (3, 3), (12, 4)])
+def test_routed_experts_alone(tmp_path, experts, top):
+    """The scores of a softmax over all experts, not renormalized: with one expert a token the
+    output is scaled by a score below one, which a renormalized router would lose."""
+    torch.manual_seed(5)
+    T, W_, ff = 33, 40, 24
+    t = {"x": torch.randn(T, W_), "router": torch.randn(experts, W_) * 0.5}
+    names = {"router": "router"}
+    for e in range(experts):
+        t[f"e{e}.up"], t[f"e{e}.down"] = torch.randn(ff, W_) * 0.3, torch.randn(W_, ff) * 0.3
+        names[f"up.{e}"], names[f"down.{e}"] = f"e{e}.up", f"e{e}.down"
+    params = {"width": W_, "ff": ff, "experts": experts, "top": top, "score": "softmax", "renormalize": False, "weight_on": "output",
+              "gated": False, "activation": "relu2"}
+    got, lm = run_alone(tmp_path, {"width": W_, "rows": T, "ffn": {"kind": "routed_experts", "params": params, "tensors": names}}, t)
+    Wd = {k: v.double() for k, v in t.items()}
+    f = {"router": {"experts": experts, "top": top}}
+    assert_close_f32(got, Wd["x"] + plain.routed_experts(Wd["x"], f, Wd, ""), "routed experts alone")
+    assert lm.paths()["routed_experts"] > 0
+
+
+def test_token_input_and_depth_mixture_alone(tmp_path):
+    """No mixer and no feed-forward: the stream gains the normed, gated row of the token table (the
+    block's own columns of it), and what the block hands on is a weighted sum of its input and its result."""
+    torch.manual_seed(6)
+    T, W_, dim, offset, eps = 27, 36, 6, 12, 1e-4
+    t = {"x": torch.randn(T, W_), "side.embed": torch.randn(T, 30), "gate": torch.randn(dim, W_) * 0.4, "proj": torch.randn(W_, dim) * 0.4,
+         "norm": 1 + 0.3 * torch.randn(W_), "dwa": torch.tensor([0.4, 1.3])}
+    cfg = {"width": W_, "rows": T,
+           "token_input": {"kind": "gated_table", "params": {"width": W_, "vocab": T, "dim": dim, "offset": offset, "table_width": 30, "eps": eps},
+                           "tensors": {"table": "side.embed", "gate": "gate", "proj": "proj", "norm": "norm"}},
+           "depth_mix": {"kind": "weighted_history", "params": {"entries": 2}, "tensors": {"weights": "dwa"}}}
+    got, _ = run_alone(tmp_path, cfg, t)
+    Wd = {k: v.double() for k, v in t.items()}
+    e = Wd["side.embed"][:, offset:offset + dim]
+    y = (plain.gelu_tanh(Wd["x"] @ Wd["gate"].T) * e) @ Wd["proj"].T
+    result = Wd["x"] + plain.rms_norm(y, Wd["norm"], eps)
+    assert_close_f32(got, 0.4 * Wd["x"] + 1.3 * result, "token input and mixture over depth alone")
