@@ -202,7 +202,7 @@ int celeg_lru_gates(const void* x, int ldx, int dtype, const float* conv_w, cons
                     const int* positions, const int* token_seq, const int* seq_start, const int* token_slot, float* decay,
                     float* input, int n_tokens, int width, int blocks, int taps, float decay_scale, hipStream_t stream);
 int celeg_lru_scan(const float* decay, const float* input, const void* y, int ldy, int dtype, float* state, size_t state_stride,
-                   const int* cu_seqlens, const int* seq_slot, void* out, int ldo, int n_seqs, int width, hipStream_t stream);
+                   const int* cu_seqlens, const int* seq_slot, void* out, int ldo, int n_seqs, int width, int longest, hipStream_t stream);
 int celeg_channel_decay(const void* z, int ldz, int dtype, const float* a_log, const float* dt_bias, float* decay, int n_tokens,
                         int heads, int dim, hipStream_t stream);
 int celeg_gla_prepare(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const void* z, int ldz, int dtype,

@@ -980,7 +980,7 @@ void Ops::lru_scan(const Tensor& decay, const Tensor& input, const Tensor& y, co
     need(state.ndim == 2 && state.shape[1] == W && state.stride[1] == 1, "lru_scan: state must be [slots, width]");
     kernel_check(celeg_lru_scan(decay.as<float>(), input.as<float>(), y.data, rows_of(y, "y"), dt(y, "y"), state.as<float>(),
                                 static_cast<size_t>(state.stride[0]), batch.cu_seqlens, batch.seq_slot, out.data, rows_of(out, "out"),
-                                batch.n_seqs, static_cast<int>(W), stream), "lru_scan");
+                                batch.n_seqs, static_cast<int>(W), batch.max_seg_len, stream), "lru_scan");
 }
 
 // ---------------------------------------------------------------------------- attention with a distance bias

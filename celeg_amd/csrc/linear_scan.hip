@@ -102,6 +102,69 @@ __global__ void lru_scan_kernel(const float* __restrict__ decay, const float* __
     *mine = S;
 }
 
+// The same recurrence for long portions, a workgroup of LRU_WAVES wavefronts per (request, 64
+// channels): a portion is taken in stretches of LRU_WAVES * LRU_CHUNK rows, a wavefront LRU_CHUNK
+// neighbouring rows of each.  A wavefront first runs its rows from S = 0, which gives its stretch as
+// a map S -> A S + L (A the product of its decays); the maps meet in LDS, every wavefront applies
+// those before its own to the state the stretch started from, in their order, and runs its rows
+// again from there.  (Sums taken in another order than token by token: the results agree to
+// rounding, not to the bit.)
+#define LRU_WAVES 16
+#define LRU_CHUNK 16
+template <typename T>
+__global__ __launch_bounds__(LRU_WAVES * CELEG_WAVE) void lru_scan_waves_kernel(
+    const float* __restrict__ decay, const float* __restrict__ input, const T* __restrict__ y, int ldy, float* __restrict__ state,
+    size_t state_stride, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_slot, T* __restrict__ out, int ldo, int width) {
+    __shared__ float prod_s[LRU_WAVES][CELEG_WAVE], last_s[LRU_WAVES][CELEG_WAVE];
+    const int s = blockIdx.y, lane = threadIdx.x % CELEG_WAVE, wave = threadIdx.x / CELEG_WAVE;
+    const int c = blockIdx.x * CELEG_WAVE + lane;
+    const bool has = c < width;
+    const int cc = has ? c : width - 1;       // lanes past the last channel repeat it and store nothing
+    const int row0 = cu_seqlens[s], n = cu_seqlens[s + 1] - row0;
+    if (n <= 0) return;
+    float* mine = state + static_cast<size_t>(seq_slot[s]) * state_stride + cc;
+    float carried = *mine;
+    for (int base = 0; base < n; base += LRU_WAVES * LRU_CHUNK) {
+        const int first = base + wave * LRU_CHUNK, count = min(LRU_CHUNK, n - first);      // <= 0: no rows here
+        float a[LRU_CHUNK], in[LRU_CHUNK], yv[LRU_CHUNK];
+#pragma unroll
+        for (int k = 0; k < LRU_CHUNK; ++k) {
+            a[k] = 1.f;
+            in[k] = 0.f;
+            yv[k] = 0.f;
+            if (k < count) {
+                const size_t t = static_cast<size_t>(row0 + first + k);
+                a[k] = decay[t * width + cc];
+                in[k] = input[t * width + cc];
+                yv[k] = to_float(y[t * ldy + cc]);
+            }
+        }
+        float A = 1.f, L = 0.f;
+#pragma unroll
+        for (int k = 0; k < LRU_CHUNK; ++k) {
+            L = fmaf(a[k], L, in[k]);
+            A *= a[k];
+        }
+        prod_s[wave][lane] = A;
+        last_s[wave][lane] = L;
+        __syncthreads();
+        float S = carried, after = carried;
+#pragma unroll
+        for (int w = 0; w < LRU_WAVES; ++w) {
+            after = fmaf(prod_s[w][lane], after, last_s[w][lane]);
+            if (w + 1 == wave) S = after;
+        }
+#pragma unroll
+        for (int k = 0; k < LRU_CHUNK; ++k) {
+            S = fmaf(a[k], S, in[k]);
+            if (has && k < count) out[static_cast<size_t>(row0 + first + k) * ldo + c] = from_float<T>(S * ls_gelu_tanh(yv[k]));
+        }
+        carried = after;
+        __syncthreads();
+    }
+    if (wave == 0 && has) *mine = carried;
+}
+
 // ---------------------------------------------------------------- decays per key channel
 // decay = exp(-exp(a_log[h]) softplus(z + dt_bias)), z [rows, heads * dim]
 template <typename T>
@@ -220,8 +283,11 @@ __global__ __launch_bounds__(CELEG_WAVE) void channel_scan_kernel(
 // The same recurrence for dim = DL * DPL (DPL a multiple of 4): DL neighbouring lanes share a column
 // of S, each holding DPL neighbouring values of it, so the sums over dim meet by log2(DL) exchanges
 // through the vector unit's cross-lane modifiers.  A request's rows are taken in blocks of TB
-// tokens whose q, k and decays are staged in LDS (asked for from memory while the block before is
-// computed) and whose values sit in registers; a token's steps wait for LDS, never for memory.
+// tokens whose q, k, decays and values are staged in LDS, asked for from memory while the block
+// before is computed: a token's steps wait for LDS, never for memory.  A wavefront issues its
+// instructions one after the other, so what a block costs besides the recurrence is kept small:
+// every lane brings pieces of four numbers whose place in the block never changes (offsets worked
+// out once; rows past the request's end read its last row again).
 // Tokens are taken one at a time in every block, so the cut of a prompt into steps changes no bit.
 template <int DL, int DPL, bool BETA>
 __global__ __launch_bounds__(CELEG_WAVE) void channel_scan_block_kernel(
@@ -229,12 +295,14 @@ __global__ __launch_bounds__(CELEG_WAVE) void channel_scan_block_kernel(
     int ld_beta, float* __restrict__ state, size_t state_stride, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_slot, float* __restrict__ out, int G, int H, int V) {
     constexpr int D = DL * DPL, NC = DPL / 4, CPW = CELEG_WAVE / DL, TB = D <= 64 ? 16 : 8, ROW = 3 * D;
-    constexpr int PER_LANE = TB * ROW / CELEG_WAVE;
+    constexpr int D4 = D / 4, PER = TB * D4 / CELEG_WAVE, PERV = (TB * CPW + CELEG_WAVE - 1) / CELEG_WAVE;
+    static_assert(TB * D4 % CELEG_WAVE == 0, "a block's pieces fill whole wavefronts");
     typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ __attribute__((aligned(16))) float rows_s[TB * ROW];
+    __shared__ float vals_s[PERV * CELEG_WAVE];
     __shared__ float beta_s[TB];
     const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int sub = lane % DL, j = blockIdx.z * CPW + lane / DL;
+    const int sub = lane % DL, col = lane / DL, j = blockIdx.z * CPW + col;
     const bool live = j < V;
     const int jj = live ? j : V - 1;          // idle lanes repeat the last column and store nothing
     const int g = h / (H / G);
@@ -244,38 +312,53 @@ __global__ __launch_bounds__(CELEG_WAVE) void channel_scan_block_kernel(
     float S[DPL];
 #pragma unroll
     for (int i = 0; i < DPL; ++i) S[i] = mine[static_cast<size_t>(sub * DPL + i) * V + jj];
-    const size_t ldqk = static_cast<size_t>(2) * G * D, ldv = static_cast<size_t>(H) * V, ldd = static_cast<size_t>(H) * D;
-    float pre[PER_LANE], pre_v[TB], pre_b = 1.f;
-    auto fetch = [&](int block) __attribute__((always_inline)) {
-        const int t0 = block * TB;
+    const int ldqk = 2 * G * D, ldv = H * V, ldd = H * D;
+    const float* q_base = qk + static_cast<size_t>(row0) * ldqk + g * D;
+    const float* k_base = q_base + G * D;
+    const float* a_base = decay + static_cast<size_t>(row0) * ldd + h * D;
+    const float* v_base = v + static_cast<size_t>(row0) * ldv + static_cast<size_t>(h) * V;
+    f4 pre_q[PER], pre_k[PER], pre_a[PER];
+    float pre_v[PERV], pre_b = 1.f;
+    auto fetch = [&](int t0) __attribute__((always_inline)) {
+        const int last = n - 1 - t0;          // the block's rows past this one read it again
 #pragma unroll
-        for (int i = 0; i < PER_LANE; ++i) {
-            const int e = lane + CELEG_WAVE * i, tt = e / ROW, x = e % ROW;
-            pre[i] = 0.f;
-            if (t0 + tt < n) {
-                const size_t t = static_cast<size_t>(row0 + t0 + tt);
-                pre[i] = x < D ? qk[t * ldqk + g * D + x] : x < 2 * D ? qk[t * ldqk + (G + g) * D + x - D] : decay[t * ldd + h * D + x - 2 * D];
-            }
+        for (int i = 0; i < PER; ++i) {
+            const int piece = lane + CELEG_WAVE * i, tt = min(piece / D4, last), c = 4 * (piece % D4);
+            const size_t t = static_cast<size_t>(t0 + tt);
+            pre_q[i] = *reinterpret_cast<const f4*>(q_base + t * ldqk + c);
+            pre_k[i] = *reinterpret_cast<const f4*>(k_base + t * ldqk + c);
+            pre_a[i] = *reinterpret_cast<const f4*>(a_base + t * ldd + c);
         }
 #pragma unroll
-        for (int tt = 0; tt < TB; ++tt) pre_v[tt] = t0 + tt < n ? v[static_cast<size_t>(row0 + t0 + tt) * ldv + static_cast<size_t>(h) * V + jj] : 0.f;
-        if (BETA && lane < TB && t0 + lane < n) pre_b = beta[static_cast<size_t>(row0 + t0 + lane) * ld_beta + h];
+        for (int i = 0; i < PERV; ++i) {
+            const int piece = lane + CELEG_WAVE * i, tt = min(piece / CPW, min(TB - 1, last));
+            const int column = min(static_cast<int>(blockIdx.z) * CPW + piece % CPW, V - 1);
+            pre_v[i] = v_base[static_cast<size_t>(t0 + tt) * ldv + column];
+        }
+        if (BETA && lane < TB) pre_b = beta[static_cast<size_t>(row0 + t0 + min(lane, last)) * ld_beta + h];
     };
     fetch(0);
-    const int n_blocks = (n + TB - 1) / TB;
-    for (int block = 0; block < n_blocks; ++block) {
+    float* out_at = out + static_cast<size_t>(row0) * ldv + static_cast<size_t>(h) * V + jj;
+    const bool stores = live && sub == 0;
+    for (int t0 = 0; t0 < n; t0 += TB) {
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < PER_LANE; ++i) rows_s[lane + CELEG_WAVE * i] = pre[i];
+        for (int i = 0; i < PER; ++i) {
+            const int piece = lane + CELEG_WAVE * i;
+            float* at = rows_s + (piece / D4) * ROW + 4 * (piece % D4);
+            *reinterpret_cast<f4*>(at) = pre_q[i];
+            *reinterpret_cast<f4*>(at + D) = pre_k[i];
+            *reinterpret_cast<f4*>(at + 2 * D) = pre_a[i];
+        }
+#pragma unroll
+        for (int i = 0; i < PERV; ++i) vals_s[lane + CELEG_WAVE * i] = pre_v[i];
         if (BETA && lane < TB) beta_s[lane] = pre_b;
-        float vals[TB];
-#pragma unroll
-        for (int tt = 0; tt < TB; ++tt) vals[tt] = pre_v[tt];
         __syncthreads();
-        if (block + 1 < n_blocks) fetch(block + 1);
-        const int count = min(TB, n - block * TB);
-        auto token = [&](int tt, float value) __attribute__((always_inline)) {
+        if (t0 + TB < n) fetch(t0 + TB);
+        const int count = min(TB, n - t0);
+        auto token = [&](int tt) __attribute__((always_inline)) {
             const float* row = rows_s + tt * ROW + sub * DPL;
+            const float value = vals_s[tt * CPW + col];
             f4 q4[NC], k4[NC], a4[NC];
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
@@ -309,15 +392,13 @@ __global__ __launch_bounds__(CELEG_WAVE) void channel_scan_block_kernel(
                     opart[e] = fmaf(q4[c][e], S[4 * c + e], opart[e]);
                 }
             const float o = lanes_sum<DL>((opart[0] + opart[1]) + (opart[2] + opart[3]));
-            if (live && sub == 0) out[static_cast<size_t>(row0 + block * TB + tt) * ldv + static_cast<size_t>(h) * V + j] = o;
+            if (stores) out_at[static_cast<size_t>(t0 + tt) * ldv] = o;
         };
         if (count == TB) {
 #pragma unroll
-            for (int tt = 0; tt < TB; ++tt) token(tt, vals[tt]);
+            for (int tt = 0; tt < TB; ++tt) token(tt);
         } else {
-#pragma unroll
-            for (int tt = 0; tt < TB; ++tt)
-                if (tt < count) token(tt, vals[tt]);
+            for (int tt = 0; tt < count; ++tt) token(tt);
         }
     }
     if (live) {
@@ -352,9 +433,20 @@ extern "C" int celeg_lru_gates(const void* x, int ldx, int dtype, const float* c
 
 extern "C" int celeg_lru_scan(const float* decay, const float* input, const void* y, int ldy, int dtype, float* state,
                               size_t state_stride, const int* cu_seqlens, const int* seq_slot, void* out, int ldo, int n_seqs,
-                              int width, hipStream_t stream) {
+                              int width, int longest, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     dim3 grid((width + 63) / 64, n_seqs), block(64);
+    // `longest`: the most rows a request has in this step; long portions are shared out over wavefronts
+    if (longest >= 4 * LRU_CHUNK) {
+        dim3 wide(LRU_WAVES * CELEG_WAVE);
+        if (dtype == CELEG_F32)
+            hipLaunchKernelGGL(lru_scan_waves_kernel<float>, grid, wide, 0, stream, decay, input, static_cast<const float*>(y), ldy, state,
+                               state_stride, cu_seqlens, seq_slot, static_cast<float*>(out), ldo, width);
+        else
+            hipLaunchKernelGGL(lru_scan_waves_kernel<bf16>, grid, wide, 0, stream, decay, input, static_cast<const bf16*>(y), ldy, state,
+                               state_stride, cu_seqlens, seq_slot, static_cast<bf16*>(out), ldo, width);
+        return CELEG_LAUNCH_RESULT();
+    }
     if (dtype == CELEG_F32)
         hipLaunchKernelGGL(lru_scan_kernel<float>, grid, block, 0, stream, decay, input, static_cast<const float*>(y), ldy, state,
                            state_stride, cu_seqlens, seq_slot, static_cast<float*>(out), ldo, width);
@@ -413,7 +505,8 @@ extern "C" int celeg_channel_scan(const float* qk, const float* v, const float* 
         return CELEG_LAUNCH_RESULT();                                                                                             \
     }
     // dims that are DL lanes of a multiple of four values each; any other dim, and `general`, take the kernel below
-    if (!general) {
+    const bool by_fours = ((reinterpret_cast<uintptr_t>(qk) | reinterpret_cast<uintptr_t>(decay)) & 15) == 0;      // the block kernel reads four numbers at a time
+    if (!general && by_fours) {
         if (D == 16) CELEG_CHANNEL_BLOCKS(4, 4)
         if (D == 32) CELEG_CHANNEL_BLOCKS(8, 4)
         if (D == 48) CELEG_CHANNEL_BLOCKS(4, 12)

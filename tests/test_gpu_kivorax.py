@@ -506,7 +506,7 @@ def test_linear_recurrent_unit_alone(tmp_path, C, B, taps):
     assert lm.paths()["linear_recurrent_unit"] > 0
 
 
-def run_alone_named(tmp_path, W_, T, part, tensors, **kw):
+def run_alone_named(tmp_path, W_, T, part, tensors, cut=CUT):
     """As ``run_alone`` for parts one of whose tensors is called "x" itself: the input is the tensor "table"."""
     from celeg_amd.config import LayerSpec, ModelSpec, PartSpec, RunStep, register_architecture, registered_architectures
     if "KivoraxPartsAloneTable" not in registered_architectures():
@@ -522,10 +522,25 @@ def run_alone_named(tmp_path, W_, T, part, tensors, **kw):
     with open(os.path.join(tmp_path, "config.json"), "w") as fh:
         json.dump({"architectures": ["KivoraxPartsAloneTable"], "width": W_, "rows": T, "mixer": part}, fh)
     write_safetensors(os.path.join(tmp_path, "model.safetensors"), {k: v.float().contiguous() for k, v in tensors.items()})
-    steps = portions_schedule({"x": list(range(T))}, sizes=CUT)
-    lm = load_model(str(tmp_path), dtype="float32", device=DEV, page_tokens=16, n_pages=8, max_requests=2, max_context=128,
-                    max_batched_tokens=64)
+    steps = portions_schedule({"x": list(range(T))}, sizes=cut)
+    pages = (T + 15) // 16 + 1
+    lm = load_model(str(tmp_path), dtype="float32", device=DEV, page_tokens=16, n_pages=pages, max_requests=2, max_context=16 * pages,
+                    max_batched_tokens=max(64, max(cut)))
     return EngineDriver(lm).run(steps)["x"].double(), lm
+
+
+@pytest.mark.parametrize("C,cut", [(70, (300, 2, 28)), (256, (64, 17, 249)), (36, (330,)), (64, (63, 65, 1, 201))])
+def test_linear_recurrent_unit_long_portions(tmp_path, C, cut):
+    """Portions of 64 rows and more are shared out over the wavefronts of a workgroup, 16 rows each
+    in stretches of 256: ends inside a wavefront's rows, inside a stretch and at their borders, and
+    the state handed from a portion taken that way to one taken token by token and back."""
+    T, W_ = 330, 40
+    t, m, part = lru_case(T, W_, C, 2, 3, seed=11)
+    t["lam"] = t["lam"] - 3.0                   # slow decays: a stretch's start still shows at its end
+    tensors = {("table" if k == "x_in" else k): v for k, v in t.items()}
+    got, _ = run_alone_named(tmp_path, W_, T, part, tensors, cut=cut)
+    Wd = {k: v.double() for k, v in t.items()}
+    assert_close_f32(got, Wd["x_in"] + plain.gated_linear_recurrent_unit(Wd["x_in"], m, Wd, ""), "linear recurrent unit, long portions")
 
 
 def test_normed_pair_alone(tmp_path):
