@@ -6,8 +6,9 @@
 //
 // Scores are computed transposed (keys as the first operand of a 16x16x32 instruction): a lane
 // holds, of row r = lane % 16, the keys 16 kt + 4 (lane / 16) + i of each of a block's four tiles.
-// Rounded to bfloat16 two tiles' weights are the second operand of the product with the values
-// without any exchange between lanes.  The softmax runs over blocks of 64 keys with a running
+// Two tiles' weights are the second operand of the product with the values without any exchange
+// between lanes; a 32-bit weight goes into that product as two bfloat16 numbers (its rounding and
+// the rest), so the weights keep sixteen bits and more where the values have eight.  The softmax runs over blocks of 64 keys with a running
 // maximum and normaliser per row in 32-bit, everything in powers of two (log2 e is folded into the
 // scale, and r1 ln(x) log2 e = r1 log2(x)): the four lanes of a row agree on the maximum by two
 // exchanges a block and keep a sum each, which meet once at the end.
@@ -130,7 +131,7 @@ __device__ __forceinline__ void bf_block(const __bf16* ks, const __bf16* vs, con
     const float keep = bf_exp2(row.top - base);
     row.top = new_top;
     float sum = 0.f;
-    bf_bf16x4 w[4];
+    bf_bf16x4 w[4], rest[4];         // a weight as two bfloat16 numbers: its rounding, and what the rounding left
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
@@ -138,6 +139,7 @@ __device__ __forceinline__ void bf_block(const __bf16* ks, const __bf16* vs, con
             const float p = bf_exp2(sacc[kt][i] - base);
             sum += p;
             w[kt][i] = static_cast<__bf16>(p);
+            rest[kt][i] = static_cast<__bf16>(p - static_cast<float>(w[kt][i]));
         }
     row.sum = fmaf(row.sum, keep, sum);
 #pragma unroll
@@ -148,13 +150,17 @@ __device__ __forceinline__ void bf_block(const __bf16* ks, const __bf16* vs, con
 #pragma unroll
     for (int pair = 0; pair < 2; ++pair) {
         const bf_bf16x8 pw = __builtin_shufflevector(w[2 * pair], w[2 * pair + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+        const bf_bf16x8 pr = __builtin_shufflevector(rest[2 * pair], rest[2 * pair + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+        bf_bf16x8 vf[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const __bf16* vrow = vs + (16 * dt + r) * VROW + 32 * pair + 4 * quad;
             const bf_u32x2 lo = *reinterpret_cast<const bf_u32x2*>(vrow), hi = *reinterpret_cast<const bf_u32x2*>(vrow + 16);
-            const bf_bf16x8 vf = __builtin_bit_cast(bf_bf16x8, bf_u32x4{lo[0], lo[1], hi[0], hi[1]});
-            row.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pw, row.acc[dt], 0, 0, 0);
+            vf[dt] = __builtin_bit_cast(bf_bf16x8, bf_u32x4{lo[0], lo[1], hi[0], hi[1]});
+            row.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pw, row.acc[dt], 0, 0, 0);
         }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) row.acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pr, row.acc[dt], 0, 0, 0);
     }
 }
 
