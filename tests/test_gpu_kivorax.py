@@ -213,6 +213,64 @@ def test_batches_of_unequal_requests_equal_each_alone(folders):
         assert float((alone[rid] - mixed[rid]).abs().max()) <= 2e-5 * float(alone[rid].abs().max()), rid
 
 
+def drawn_model(rng):
+    """A configuration drawn at random: widths, head counts and sizes (those the kernels in registers and on
+    the matrix cores take, and others), order and number of layers, feed-forwards and constants."""
+    cfg = {"architecture": "Kivorax", "vocab": rng.randint(100, 700), "width": rng.choice([64, 96, 160, 192, 224, 320]),
+           "norm": {"eps": rng.choice([1e-6, 1e-5])}}
+    if rng.random() < 0.8:
+        cfg["embedding"] = {"scale": round(rng.uniform(0.5, 4.0), 3)}
+    if rng.random() < 0.8:
+        cfg["token_side"] = {"dim": rng.choice([4, 8, 16, 24, 32])}
+
+    def mlp():
+        r = rng.random()
+        if r < 0.15:
+            return None
+        if r < 0.45:
+            return dense(rng.choice([64, 200, 256]))
+        experts = rng.choice([2, 4, 8, 12, 16])
+        return moe(experts, rng.randint(1, min(4, experts)), rng.choice([32, 64, 96]))
+    layers = []
+    for _ in range(rng.randint(3, 7)):
+        kind = rng.choice("pdg")
+        if kind == "p":
+            kv, dim, inner = rng.choice([1, 2, 3, 4]), rng.choice([16, 32, 48, 64, 80, 128, 160]), rng.choice([32, 96, 160, 256, 384])
+            q_temp = (round(rng.uniform(0.1, 0.5), 3), rng.choice([1, 8, 64, 128, 256])) if rng.random() < 0.8 else None
+            layers.append(pair(kv * rng.choice([1, 2, 3, 4]), kv, dim, rng.choice([16, 32, 64, 96, 128, 192]),
+                               round(dim ** -0.5 * rng.uniform(0.7, 1.5), 4), q_temp, inner, rng.choice([1, 2, 4, 8]),
+                               rng.choice([2, 3, 4, 5]), mlp()))
+        elif kind == "d":
+            kv = rng.choice([1, 2, 4, 6])
+            layers.append(channel_delta(kv * rng.choice([1, 2]), kv, rng.choice([16, 24, 32, 64, 80, 128]), rng.choice([16, 32, 64, 100, 128]),
+                                        rng.choice([2, 3, 4]), mlp(), decay_rank=rng.choice([4, 16, 32]), gate_rank=rng.choice([4, 16, 32])))
+        else:
+            layers.append(gla(rng.choice([1, 2, 4, 6]), rng.choice([16, 32, 48, 64, 96]), rng.choice([16, 32, 64, 100, 128]),
+                              rng.choice([4.0, 8.0, 16.0, 32.0]), mlp(), decay_rank=rng.choice([4, 16, 32])))
+    cfg["layers"] = layers
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_models_drawn_at_random(tmp_path, seed):
+    """Eight models drawn at random, weights stored in bfloat16, four requests of 20 to 300 tokens,
+    in a mixed schedule and in long and short portions, in 32-bit and in bfloat16."""
+    import random
+    rng = random.Random(1000 + seed)
+    cfg = drawn_model(rng)
+    folder = write_model(tmp_path / "drawn", cfg, seed, torch.bfloat16, std=0.06)
+    c, W = plain.load_model_folder(folder)
+    reqs = {f"r{i}": random_tokens(cfg["vocab"], rng.randint(20, 300), seed=seed * 10 + i) for i in range(4)}
+    ref = {rid: plain.forward(c, W, toks) for rid, toks in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        for steps in (mixed_schedule(reqs, seed=seed, decode_tail=rng.randint(3, 20)), portions_schedule(reqs, sizes=(70, 2, 33, 1, 130, 16, 5))):
+            lm, _ = load(folder, dtype, steps)
+            got = EngineDriver(lm).run(steps)
+            for rid in reqs:
+                assert_close(got[rid], ref[rid], dtype, f"drawn model {seed}/{dtype}/{rid}: {json.dumps(cfg)}")
+            lm.close()
+
+
 # ------------------------------------------------------------------ inputs made so that a fault shows
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_state_that_remembers_hundreds_of_tokens(tmp_path, dtype):
