@@ -50,6 +50,8 @@ class LayerSpec:
     # the layer is mixed from the results of all entries of the run order so far
     token_input: Optional[PartSpec] = None
     depth_mix: Optional[PartSpec] = None
+    # what a sub-layer's (normed) output is multiplied by as it is added to the stream ("sandwich_norm")
+    residual_scale: float = 1.0
 
     def to_json(self) -> Dict[str, Any]:
         out = {"mixer": self.mixer.to_json(), "mixer_norm": self.mixer_norm.to_json(),
@@ -67,6 +69,8 @@ class LayerSpec:
             out["token_input"] = self.token_input.to_json()
         if self.depth_mix is not None:
             out["depth_mix"] = self.depth_mix.to_json()
+        if self.residual_scale != 1.0:
+            out["residual_scale"] = self.residual_scale
         return out
 
     @classmethod
@@ -75,7 +79,8 @@ class LayerSpec:
         return cls(PartSpec.from_json(l["mixer"]), PartSpec.from_json(l["mixer_norm"]),
                    PartSpec.from_json(l["ffn"]), PartSpec.from_json(l["ffn_norm"]),
                    l.get("arrangement", "pre_norm"), link("mixer_link"), link("ffn_link"),
-                   link("mixer_post_norm"), link("ffn_post_norm"), link("token_input"), link("depth_mix"))
+                   link("mixer_post_norm"), link("ffn_post_norm"), link("token_input"), link("depth_mix"),
+                   float(l.get("residual_scale", 1.0)))
 
 
 @dataclass(frozen=True)
@@ -84,10 +89,12 @@ class RunStep:
     more than once: its weights are shared, its cache is not).  ``kv_from`` is the index of an
     EARLIER entry of the run order whose keys and values this entry's mixer reads instead of
     writing its own.  ``reinject``: before this entry the stream is replaced by the model's
-    ``reinjection`` part's mixture of the stream and the embedding's rows."""
+    ``reinjection`` part's mixture of the stream and the embedding's rows.  ``pass_``: which run
+    of a looped range of layers the entry belongs to ("pass" in JSON)."""
     layer: int
     kv_from: Optional[int] = None
     reinject: bool = False
+    pass_: int = 0
 
 
 @dataclass(frozen=True)
@@ -111,15 +118,15 @@ class ModelSpec:
         return {**out, "architecture": self.architecture, "vocab_size": self.vocab_size,
                 "hidden_size": self.hidden_size, "max_context": self.max_context, "streams": self.streams,
                 "embedding": self.embedding.to_json(), "layers": [l.to_json() for l in self.layers],
-                "order": [{"layer": s.layer, "kv_from": s.kv_from, **({"reinject": True} if s.reinject else {})}
-                          for s in self.order],
+                "order": [{"layer": s.layer, "kv_from": s.kv_from, **({"reinject": True} if s.reinject else {}),
+                           **({"pass": s.pass_} if s.pass_ else {})} for s in self.order],
                 "final_norm": self.final_norm.to_json(), "head": self.head.to_json(),
                 "eos_token_ids": list(self.eos_token_ids), "bos_token_id": self.bos_token_id}
 
     @classmethod
     def from_json(cls, j: Dict[str, Any]) -> "ModelSpec":
         layers = tuple(LayerSpec.from_json(l) for l in j["layers"])
-        order = tuple(RunStep(s["layer"], s.get("kv_from"), bool(s.get("reinject"))) for s in j["order"])
+        order = tuple(RunStep(s["layer"], s.get("kv_from"), bool(s.get("reinject")), int(s.get("pass") or 0)) for s in j["order"])
         return cls(j["architecture"], j["vocab_size"], j["hidden_size"], j["max_context"],
                    PartSpec.from_json(j["embedding"]), layers, order, PartSpec.from_json(j["final_norm"]),
                    PartSpec.from_json(j["head"]), tuple(j.get("eos_token_ids") or ()), j.get("bos_token_id"),

@@ -2,7 +2,9 @@
 //     score(i, j) = (q_i . k_j) * scale * f(i) - r1[h] * ln(1 + r2[h] * (i - j))
 // with a factor per query position f(i) = 1 + coef * ln(floor((i + 1) / every) + 1) (or 1) and a
 // distance bias per query head (or none).  Keys at positions [first, i] of the row's request,
-// first = max(0, i - window + 1) with a window, else 0.  Values may be wider or narrower than keys.
+// first = max(0, i - window + 1) with a window, else 0; with `keep_first` the keys at positions
+// [0, keep_first) stay visible after the window has passed them.  `sink_one`: the softmax's denominator
+// holds a one more (a key whose score is 0 and that has no value).  Values may be wider or narrower than keys.
 //
 // Cache layout: K [pages, layers, kv_heads, page_tokens, head_dim],
 // V [pages, layers, kv_heads, v_dim, page_tokens].
@@ -51,7 +53,8 @@ __global__ __launch_bounds__(CELEG_WAVE) void biased_attention_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool, const int* __restrict__ table,
     int table_stride, const int* __restrict__ token_slot, const int* __restrict__ positions, const float* __restrict__ r1,
     const float* __restrict__ r2, const T* __restrict__ gate, int ldg, T* __restrict__ out, int ldo, int q_heads, int kv_heads,
-    int head_dim, int v_dim, int page_tokens, int n_layers, int layer, float scale, float coef, int every, int window) {
+    int head_dim, int v_dim, int page_tokens, int n_layers, int layer, float scale, float coef, int every, int window,
+    int keep_first, int sink_one) {
     extern __shared__ float lds[];  // head_dim floats of q, then 64 weights
     float* qs = lds;
     float* ps = lds + head_dim;
@@ -70,12 +73,17 @@ __global__ __launch_bounds__(CELEG_WAVE) void biased_attention_kernel(
     float acc[BA_MAX_V_CHUNKS];
 #pragma unroll
     for (int j = 0; j < BA_MAX_V_CHUNKS; ++j) acc[j] = 0.f;
-    float top = -INFINITY, total = 0.f;
+    // (the extra one of the denominator: a key of score 0 seen before all others)
+    float top = sink_one ? 0.f : -INFINITY, total = sink_one ? 1.f : 0.f;
 
-    for (int base = first; base <= pos; base += CELEG_WAVE) {
+    // the kept first keys that the window has passed, then the window (or everything)
+    const int kept = min(keep_first, first);
+    for (int phase = kept > 0 ? 0 : 1; phase < 2; ++phase) {
+    const int lo = phase == 0 ? 0 : first, hi = phase == 0 ? kept - 1 : pos;
+    for (int base = lo; base <= hi; base += CELEG_WAVE) {
         const int key = base + lane;
         float score = -INFINITY;
-        if (key <= pos) {
+        if (key <= hi) {
             const T* kp = k_pool + ba_k_offset(pages[key / page_tokens], n_layers, layer, kv_heads, kvh, page_tokens,
                                                key % page_tokens, head_dim);
             float dot = 0.f;
@@ -84,13 +92,13 @@ __global__ __launch_bounds__(CELEG_WAVE) void biased_attention_kernel(
             if (r1) score -= b1 * logf(1.0f + b2 * static_cast<float>(pos - key));
         }
         const float new_top = fmaxf(top, wave_max(score));     // (the round holds at least one visible key)
-        const float p = key <= pos ? expf(score - new_top) : 0.f;
+        const float p = key <= hi ? expf(score - new_top) : 0.f;
         const float keep = expf(top - new_top);                // 0 in the first round
         total = total * keep + wave_sum(p);
         top = new_top;
         ps[lane] = p;
         __syncthreads();
-        const int n_keys = min(CELEG_WAVE, pos - base + 1);
+        const int n_keys = min(CELEG_WAVE, hi - base + 1);
 #pragma unroll
         for (int j = 0; j < BA_MAX_V_CHUNKS; ++j) acc[j] *= keep;
         for (int kk = 0; kk < n_keys; ++kk) {
@@ -105,6 +113,7 @@ __global__ __launch_bounds__(CELEG_WAVE) void biased_attention_kernel(
             }
         }
         __syncthreads();
+    }
     }
     const float inv = 1.0f / total;
     T* orow = out + static_cast<size_t>(t) * ldo + static_cast<size_t>(h) * v_dim;
@@ -145,7 +154,7 @@ extern "C" int celeg_biased_attention(const void* q, int ldq, int dtype, const v
                                       int table_stride, const int* token_slot, const int* positions, const float* r1,
                                       const float* r2, const void* gate, int ldg, void* out, int ldo, int n_tokens, int q_heads,
                                       int kv_heads, int head_dim, int v_dim, int page_tokens, int n_layers, int layer, float scale,
-                                      float coef, int every, int window, hipStream_t stream) {
+                                      float coef, int every, int window, int keep_first, int sink_one, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (v_dim > BA_MAX_V_CHUNKS * CELEG_WAVE || q_heads % kv_heads) return static_cast<int>(hipErrorInvalidValue);
     dim3 grid(n_tokens, q_heads), block(CELEG_WAVE);
@@ -154,11 +163,11 @@ extern "C" int celeg_biased_attention(const void* q, int ldq, int dtype, const v
         hipLaunchKernelGGL(biased_attention_kernel<float>, grid, block, lds, stream, static_cast<const float*>(q), ldq,
                            static_cast<const float*>(k_pool), static_cast<const float*>(v_pool), table, table_stride, token_slot,
                            positions, r1, r2, static_cast<const float*>(gate), ldg, static_cast<float*>(out), ldo, q_heads,
-                           kv_heads, head_dim, v_dim, page_tokens, n_layers, layer, scale, coef, every, window);
+                           kv_heads, head_dim, v_dim, page_tokens, n_layers, layer, scale, coef, every, window, keep_first, sink_one);
     else
         hipLaunchKernelGGL(biased_attention_kernel<bf16>, grid, block, lds, stream, static_cast<const bf16*>(q), ldq,
                            static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool), table, table_stride, token_slot,
                            positions, r1, r2, static_cast<const bf16*>(gate), ldg, static_cast<bf16*>(out), ldo, q_heads, kv_heads,
-                           head_dim, v_dim, page_tokens, n_layers, layer, scale, coef, every, window);
+                           head_dim, v_dim, page_tokens, n_layers, layer, scale, coef, every, window, keep_first, sink_one);
     return CELEG_LAUNCH_RESULT();
 }

@@ -1,6 +1,8 @@
 // Softmax attention with a factor per query position and a distance bias per head, bfloat16, on
 // the matrix cores:
 //     score(i, j) = (q_i . k_j) * scale * f(i) - r1[h] * ln(1 + r2[h] * (i - j)),   weights = softmax over the visible j
+// Visible: j <= i, inside the window where there is one, or among the first `keep_first` positions.  With `sink_one`
+// the denominator holds a one more (a key of score 0 without a value, which the row meets before all others).
 // Keys of `D` numbers, values of `V` numbers a head (both multiples of 32 up to 128).
 // Cache layout: K [pages, layers, kv_heads, page_tokens, D], V [pages, layers, kv_heads, V, page_tokens].
 //
@@ -99,7 +101,8 @@ struct BfFetch {
 // one staged block of 64 keys for the 16 rows of a wavefront
 template <int D, int V>
 __device__ __forceinline__ void bf_block(const __bf16* ks, const __bf16* vs, const bf_bf16x8 (&qreg)[D / 32], BfRow<V / 16>& row, int kb,
-                                         int my_pos, int window, int r, int quad, float s2, float b1, float b2, bool biased) {
+                                         int my_pos, int window, int keep_first, bool kept_only, int r, int quad, float s2, float b1, float b2,
+                                         bool biased) {
     constexpr int KROW = D + 8, VROW = BF_KEYS + 8, KS = D / 32, DT = V / 16;
     bf_f32x4 sacc[4];
 #pragma unroll
@@ -117,7 +120,7 @@ __device__ __forceinline__ void bf_block(const __bf16* ks, const __bf16* vs, con
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int key = kb + 16 * kt + 4 * quad + i;
-            const bool seen = key <= my_pos && (window <= 0 || key > my_pos - window);
+            const bool seen = key <= my_pos && (kept_only ? key < keep_first : (window <= 0 || key > my_pos - window || key < keep_first));
             float x = sacc[kt][i] * s2;
             if (biased) x -= b1 * bf_log2(fmaf(b2, static_cast<float>(my_pos - key), 1.0f));
             x = seen ? x : -INFINITY;
@@ -195,8 +198,28 @@ struct BfArgs {
     const float* r2;
     const bf16* gate;
     bf16* out;
-    int ldq, ldg, ldo, table_stride, n_seqs, q_heads, kv_heads, page_tokens, n_layers, layer, every, window;
+    int ldq, ldg, ldo, table_stride, n_seqs, q_heads, kv_heads, page_tokens, n_layers, layer, every, window, keep_first, sink_one;
     float scale, coef;
+};
+
+// The key blocks of a tile whose lowest position is pos0: first the blocks that hold the kept first keys
+// where the window has passed them (only those keys count there), then the blocks from the window's start on.
+struct BfBlocks {
+    int n_kept, kb0;
+    __device__ __forceinline__ BfBlocks(int pos0, int window, int keep) {
+        const int key_first = window > 0 ? max(0, pos0 - window + 1) : 0;
+        kb0 = key_first & ~7;
+        n_kept = 0;
+        if (keep > 0 && kb0 > 0) {
+            if (kb0 >= keep) n_kept = (keep + BF_KEYS - 1) / BF_KEYS;
+            else kb0 = 0;                 // the window begins among the kept keys: one run from the start
+        }
+    }
+    __device__ __forceinline__ int count(int pos_last) const { return n_kept + (pos_last >= kb0 ? (pos_last - kb0) / BF_KEYS + 1 : 0); }
+    __device__ __forceinline__ bool kept(int i) const { return i < n_kept; }
+    __device__ __forceinline__ int start(int i) const { return i < n_kept ? i * BF_KEYS : kb0 + (i - n_kept) * BF_KEYS; }
+    // the last key a block may touch: pages between the kept keys and the window may be gone
+    __device__ __forceinline__ int last(int i, int pos_last, int keep) const { return i < n_kept ? keep - 1 : pos_last; }
 };
 
 // which tile of `rows` rows: tiles of all requests of the step, one after the other
@@ -240,24 +263,31 @@ __global__ __launch_bounds__(BF_WAVES * CELEG_WAVE) void biased_attention_rows_k
     BfRow<DT> row;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) row.acc[dt] = bf_f32x4{0.f, 0.f, 0.f, 0.f};
-    const int key_first = a.window > 0 ? max(0, tile_pos0 - a.window + 1) : 0;
+    if (a.sink_one) {
+        row.top = 0.f;
+        row.sum = quad == 0 ? 1.f : 0.f;
+    }
     const int page_shift = 31 - __builtin_clz(a.page_tokens), page_mask = a.page_tokens - 1;
     const size_t head_index_stride = static_cast<size_t>(a.n_layers) * a.kv_heads, layer_index = static_cast<size_t>(a.layer) * a.kv_heads;
     BfFetch<D, V, THREADS> pre;
-    const int kb0 = key_first & ~7;
-    pre.load(tid, kb0, pos_last, a.k_pool, a.v_pool, pages, page_shift, page_mask, a.page_tokens, head_index_stride, kvh, layer_index);
+    const BfBlocks blocks(tile_pos0, a.window, a.keep_first);
+    const int n_blocks = blocks.count(pos_last);
+    pre.load(tid, blocks.start(0), blocks.last(0, pos_last, a.keep_first), a.k_pool, a.v_pool, pages, page_shift, page_mask, a.page_tokens,
+             head_index_stride, kvh, layer_index);
     int turn = 0;
-    for (int kb = kb0; kb <= pos_last; kb += BF_KEYS, turn ^= 1) {
+    for (int i = 0; i < n_blocks; ++i, turn ^= 1) {
+        const int kb = blocks.start(i);
         __bf16* ks = lds + turn * BUF;
         __bf16* vs = ks + BF_KEYS * KROW;
         pre.stage(tid, ks, vs);
         __syncthreads();
-        if (kb + BF_KEYS <= pos_last)
-            pre.load(tid, kb + BF_KEYS, pos_last, a.k_pool, a.v_pool, pages, page_shift, page_mask, a.page_tokens, head_index_stride, kvh,
-                     layer_index);
+        if (i + 1 < n_blocks)
+            pre.load(tid, blocks.start(i + 1), blocks.last(i + 1, pos_last, a.keep_first), a.k_pool, a.v_pool, pages, page_shift, page_mask,
+                     a.page_tokens, head_index_stride, kvh, layer_index);
         // blocks none of this wavefront's rows can see
-        if (rows_here <= 0 || kb > wave_last || (a.window > 0 && kb + BF_KEYS - 1 < wave_pos0 - a.window + 1)) continue;
-        bf_block<D, V>(ks, vs, qreg, row, kb, my_pos, a.window, r, quad, s2, b1, b2, biased);
+        if (rows_here <= 0) continue;
+        if (!blocks.kept(i) && (kb > wave_last || (a.window > 0 && kb >= a.keep_first && kb + BF_KEYS - 1 < wave_pos0 - a.window + 1))) continue;
+        bf_block<D, V>(ks, vs, qreg, row, kb, my_pos, a.window, a.keep_first, blocks.kept(i), r, quad, s2, b1, b2, biased);
     }
     float total = row.sum;
     total += __shfl_xor(total, 16, CELEG_WAVE);
@@ -294,24 +324,29 @@ __global__ __launch_bounds__(WAVES * CELEG_WAVE) void biased_attention_tile_kern
     BfRow<DT> row;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) row.acc[dt] = bf_f32x4{0.f, 0.f, 0.f, 0.f};
-    const int key_first = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
+    if (a.sink_one && wave == 0) {        // (once a row: the first wavefront's share)
+        row.top = 0.f;
+        row.sum = quad == 0 ? 1.f : 0.f;
+    }
     const int page_shift = 31 - __builtin_clz(a.page_tokens), page_mask = a.page_tokens - 1;
     const size_t head_index_stride = static_cast<size_t>(a.n_layers) * a.kv_heads, layer_index = static_cast<size_t>(a.layer) * a.kv_heads;
     BfFetch<D, V, CELEG_WAVE> pre;
-    const int kb0 = (key_first & ~7) + wave * BF_KEYS;
-    if (kb0 <= pos_last)
-        pre.load(lane, kb0, pos_last, a.k_pool, a.v_pool, pages, page_shift, page_mask, a.page_tokens, head_index_stride, kvh, layer_index);
-    for (int kb = kb0; kb <= pos_last; kb += WAVES * BF_KEYS) {
+    const BfBlocks blocks(pos0, a.window, a.keep_first);
+    const int n_blocks = blocks.count(pos_last);
+    if (wave < n_blocks)
+        pre.load(lane, blocks.start(wave), blocks.last(wave, pos_last, a.keep_first), a.k_pool, a.v_pool, pages, page_shift, page_mask,
+                 a.page_tokens, head_index_stride, kvh, layer_index);
+    for (int i = wave; i < n_blocks; i += WAVES) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         pre.stage(lane, ks, vs);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        if (kb + WAVES * BF_KEYS <= pos_last)
-            pre.load(lane, kb + WAVES * BF_KEYS, pos_last, a.k_pool, a.v_pool, pages, page_shift, page_mask, a.page_tokens, head_index_stride,
-                     kvh, layer_index);
-        bf_block<D, V>(ks, vs, qreg, row, kb, my_pos, a.window, r, quad, s2, b1, b2, biased);
+        if (i + WAVES < n_blocks)
+            pre.load(lane, blocks.start(i + WAVES), blocks.last(i + WAVES, pos_last, a.keep_first), a.k_pool, a.v_pool, pages, page_shift,
+                     page_mask, a.page_tokens, head_index_stride, kvh, layer_index);
+        bf_block<D, V>(ks, vs, qreg, row, blocks.start(i), my_pos, a.window, a.keep_first, blocks.kept(i), r, quad, s2, b1, b2, biased);
     }
     // the wavefronts' maxima, normalisers and sums meet in LDS (every wavefront's staging area is
     // free after the barrier); the first one joins them in the order of the wavefronts and stores
@@ -401,7 +436,8 @@ extern "C" int celeg_biased_attention_fast(int form, const void* q, int ldq, con
                                            int table_stride, const int* cu_seqlens, const int* seq_slot, const int* seq_start, int n_seqs,
                                            int max_tiles, const float* r1, const float* r2, const void* gate, int ldg, void* out, int ldo,
                                            int q_heads, int kv_heads, int head_dim, int v_dim, int page_tokens, int n_layers, int layer,
-                                           float scale, float coef, int every, int window, hipStream_t stream) {
+                                           float scale, float coef, int every, int window, int keep_first, int sink_one,
+                                           hipStream_t stream) {
     if (max_tiles <= 0 || n_seqs <= 0) return 0;
     if (!celeg_biased_attention_fast_ok(head_dim, v_dim) || q_heads % kv_heads || page_tokens < 8 || (page_tokens & (page_tokens - 1)) ||
         ldq % 8 || ldo % 4 || (gate && ldg % 4) || (r1 == nullptr) != (r2 == nullptr))
@@ -430,6 +466,8 @@ extern "C" int celeg_biased_attention_fast(int form, const void* q, int ldq, con
     a.layer = layer;
     a.every = every;
     a.window = window;
+    a.keep_first = window > 0 ? keep_first : 0;
+    a.sink_one = sink_one;
     a.scale = scale;
     a.coef = coef;
     switch (head_dim) {

@@ -36,7 +36,7 @@ LINK_FLAGS = ["-shared", "-fPIC", f"--offload-arch={ARCH}", "-ldl", "-lpthread"]
 # the kernel files, by the name tests and tools know them under
 MODULES = ["elementwise", "gemm_f32", "short_conv", "attention", "attention_fast", "gemv_fused", "gemv_slices",
            "gemm_rows", "gemm_tiles", "sampling", "hyper", "latent", "latent_fast", "moe",
-           "norm_step", "sigmoid_attention", "delta_rule", "layer_glue", "biased_attention", "biased_attention_fast", "linear_scan"]
+           "norm_step", "sigmoid_attention", "delta_rule", "layer_glue", "biased_attention", "biased_attention_fast", "linear_scan", "conv_rope"]
 LIBRARY = "libceleg_amd"
 _lock = threading.Lock()
 

@@ -72,7 +72,7 @@ Json CacheLayout::to_json() const {
         groups.push(Json::object().set("kv_heads", kv_groups[g].kv_heads).set("head_dim", kv_groups[g].head_dim)
                         .set("v_head_dim", kv_groups[g].value_dim()).set("keys_only", kv_groups[g].keys_only)
                         .set("window", kv_groups[g].window ? Json(*kv_groups[g].window) : Json())
-                        .set("layers", group_layers[g]));
+                        .set("keep_first", kv_groups[g].kept()).set("layers", group_layers[g]));
     Json uses = Json::array();
     for (const auto& u : kv_of_step)
         uses.push(Json::object().set("step", u.first).set("group", u.second.group).set("layer", u.second.layer)
@@ -95,6 +95,7 @@ CacheLayout CacheLayout::from_json(const Json& j) {
             need.keys_only = g.get_bool("keys_only", false);
             if (need.v_head_dim == need.head_dim || need.keys_only) need.v_head_dim = 0;
             if (!g["window"].is_null()) need.window = static_cast<int>(g["window"].as_int());
+            need.keep_first = static_cast<int>(g.get_int("keep_first", 0));
             out.kv_groups.push_back(need);
             out.group_layers.push_back(static_cast<int>(g.get_int("layers", 1)));
         }
@@ -218,7 +219,9 @@ void CacheManager::release_passed(Group& g, int slot, int next_pos) {
     const int first_needed_page = lowest_needed / page_tokens;
     auto& pages = g.pages[static_cast<size_t>(slot)];
     const int stop = std::min(first_needed_page, static_cast<int>(pages.size()));
-    for (int idx = g.first_live[static_cast<size_t>(slot)]; idx < stop; ++idx)
+    // (the pages of the kept first positions are never among those given back)
+    const int kept_pages = (g.need.kept() + page_tokens - 1) / page_tokens;
+    for (int idx = std::max(g.first_live[static_cast<size_t>(slot)], kept_pages); idx < stop; ++idx)
         if (pages[static_cast<size_t>(idx)] >= 0) {
             g.pool.release({pages[static_cast<size_t>(idx)]});
             pages[static_cast<size_t>(idx)] = -1;
@@ -261,6 +264,9 @@ bool CacheManager::covers(int slot, int start_pos, int n_new) const {
         if (top >= static_cast<int>(pages.size())) return false;
         const int low = g.need.window ? std::max(0, start_pos - *g.need.window + 1) : 0;
         for (int idx = low / page_tokens; idx <= top; ++idx)
+            if (pages[static_cast<size_t>(idx)] < 0) return false;
+        const int kept_pages = std::min((g.need.kept() + page_tokens - 1) / page_tokens, low / page_tokens);
+        for (int idx = 0; idx < kept_pages; ++idx)
             if (pages[static_cast<size_t>(idx)] < 0) return false;
     }
     return true;

@@ -16,7 +16,8 @@
 // (null_slot) is never given to a request.
 //
 // Pages are given back when a request closes, and, in a window group, as soon as every
-// position of a page lies before the window of the next token.
+// position of a page lies before the window of the next token (pages that hold one of the first
+// `keep_first` positions stay: those keys remain visible behind the window).
 #pragma once
 #include <map>
 #include <optional>
@@ -62,10 +63,12 @@ struct KVNeed {
     std::optional<int> window;
     int v_head_dim = 0;
     bool keys_only = false;
+    int keep_first = 0;           // with a window: the sequence's first positions that stay readable
     int value_dim() const { return keys_only ? 0 : v_head_dim > 0 ? v_head_dim : head_dim; }
+    int kept() const { return window ? keep_first : 0; }
     bool operator==(const KVNeed& o) const {
         return kv_heads == o.kv_heads && head_dim == o.head_dim && window == o.window && value_dim() == o.value_dim() &&
-               keys_only == o.keys_only;
+               keys_only == o.keys_only && kept() == o.kept();
     }
 };
 

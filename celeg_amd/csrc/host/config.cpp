@@ -1061,6 +1061,270 @@ ModelSpec kivorax_build_spec(const Json& c) {
 
 }  // namespace
 
+// ---------------------------------------------------------------------------- Vabuzen
+// A decoder whose sub-layers are wrapped in "dynamic tanh" norms (tanh(alpha x) w + b, no statistics)
+// before and after, their output added times a constant; two kinds of attention; dense or routed
+// feed-forwards; a range of layers that may run several times, a learned vector of the run (and, from the
+// second run on, the embedding's rows) added to the stream before each run; logits bent by a tanh.
+// config.json describes every layer by itself:
+//   {"architecture": "Vabuzen", "vocab", "width", "norm": {"eps"}, "residual_mult" (absent: 1),
+//    "logit_softcap" (absent or null: none), "loop": {"start", "stop", "times"} (absent: none),
+//    "max_context" (an engine limit; optional),
+//    "layers": [{"type": "attention",
+//                "mixer": {"heads", "kv_heads", "dim", "vdim" (absent: dim), "scale", "conv" (taps; absent or 0: none),
+//                          "rot": {"base", "dims"} (absent, or dims 0: no rotation; neighbouring values pair),
+//                          "mask": {"size", "keep_first" (absent: 0)} (absent: every earlier key)},
+//                "mlp": null | {"kind": "dense", "ff"}
+//                            | {"kind": "moe", "expert": {"ff"}, "shared": {"ff"} (absent or null: none),
+//                               "router": {"experts", "top", "scale" (absent: 1), "groups": {"count", "keep"} (absent: one group)}}},
+//               {"type": "latent_attention",
+//                "mixer": {"heads", "dim", "rot_dim", "vdim", "kv_rank", "scale", "rot": {"base", "dims"}} (the two halves
+//                          of the rotated part pair), "mlp": ...}]}
+// The attention's softmax has a one more in its denominator; the latent attention's is the ordinary one.
+// Tensors: embed, head, loop.step [times, width], final.norm(.b, .alpha), l<i>.norm1|norm1b|norm2|norm2b(.b, .alpha),
+// attention: l<i>.mix.{q, k, v, o, q.conv, k.conv, v.conv}; latent: l<i>.mix.{q, dkv, dkv.norm, uk, uv, o};
+// l<i>.mlp.{up, up.b, down, down.b} or l<i>.mlp.router, l<i>.mlp.e<j>.{gate, up, down}, l<i>.mlp.shared.{gate, up, down}.
+namespace {
+
+Json vabuzen_rot(const Json& m, const std::string& mw, long long most, const char* most_name) {
+    if (m["rot"].is_null()) return Json();
+    const Json& r = regipel_object(m, "rot", mw);
+    const long long dims = regipel_int(r, "dims", mw + "rot.", 0);
+    if (dims % 2 || dims > most) throw ConfigError("config.json: " + mw + "'rot.dims' must be even and at most '" + most_name + "'");
+    if (dims == 0) return Json();
+    const double base = regipel_number(r, "base", mw + "rot.");
+    if (!(base > 0)) throw ConfigError("config.json: " + mw + "'rot.base' must be positive");
+    return Json::object().set("base", base).set("dims", dims);
+}
+
+Json vabuzen_read_config(const Json& raw, const TensorShapes*) {
+    if (!raw.is_object()) throw ConfigError("config.json is not an object");
+    Json out = Json::object();
+    out.set("architecture", "Vabuzen");
+    out.set("vocab", regipel_int(raw, "vocab", ""));
+    const long long width = regipel_int(raw, "width", "");
+    out.set("width", width);
+    const double eps = regipel_number(regipel_object(raw, "norm", ""), "eps", "norm.");
+    if (!(eps > 0)) throw ConfigError("config.json: 'norm.eps' must be positive");
+    out.set("norm", Json::object().set("eps", eps));
+    out.set("residual_mult", raw["residual_mult"].is_null() ? 1.0 : regipel_number(raw, "residual_mult", ""));
+    if (raw["logit_softcap"].is_null()) {
+        out.set("logit_softcap", Json());
+    } else {
+        const double cap = regipel_number(raw, "logit_softcap", "");
+        if (!(cap > 0)) throw ConfigError("config.json: 'logit_softcap' must be positive");
+        out.set("logit_softcap", cap);
+    }
+    out.set("max_context", raw["max_context"].is_null() ? 131072LL : regipel_int(raw, "max_context", ""));
+    if (!raw["layers"].is_array() || raw["layers"].size() == 0) throw ConfigError("config.json: 'layers' must be a list of layers");
+    Json layers = Json::array();
+    int i = 0;
+    for (const Json& l : raw["layers"].items()) {
+        const std::string where = "layers[" + std::to_string(i++) + "].";
+        if (!l.is_object()) throw ConfigError("config.json: " + where + " must be an object");
+        const std::string type = l.get_string("type", "");
+        const Json& m = regipel_object(l, "mixer", where);
+        const std::string mw = where + "mixer.";
+        Json mixer = Json::object();
+        const long long heads = regipel_int(m, "heads", mw), dim = regipel_int(m, "dim", mw);
+        mixer.set("heads", heads).set("dim", dim).set("scale", regipel_number(m, "scale", mw));
+        if (type == "attention") {
+            const long long kv_heads = m["kv_heads"].is_null() ? heads : regipel_int(m, "kv_heads", mw);
+            if (heads % kv_heads) throw ConfigError("config.json: " + mw + "'heads' must be a multiple of 'kv_heads'");
+            mixer.set("kv_heads", kv_heads).set("vdim", m["vdim"].is_null() ? dim : regipel_int(m, "vdim", mw));
+            mixer.set("conv", m["conv"].is_null() ? 0LL : regipel_int(m, "conv", mw, 0));
+            mixer.set("rot", vabuzen_rot(m, mw, dim, "dim"));
+            Json mask;
+            if (!m["mask"].is_null()) {
+                const Json& k = regipel_object(m, "mask", mw);
+                mask = Json::object().set("size", regipel_int(k, "size", mw + "mask."))
+                           .set("keep_first", k["keep_first"].is_null() ? 0LL : regipel_int(k, "keep_first", mw + "mask.", 0));
+            }
+            mixer.set("mask", mask);
+        } else if (type == "latent_attention") {
+            const long long rot_dim = regipel_int(m, "rot_dim", mw, 0);
+            mixer.set("rot_dim", rot_dim).set("vdim", regipel_int(m, "vdim", mw)).set("kv_rank", regipel_int(m, "kv_rank", mw));
+            mixer.set("rot", rot_dim > 0 ? vabuzen_rot(m, mw, rot_dim, "rot_dim") : Json());
+        } else {
+            throw ConfigError("config.json: " + where + "'type' is '" + type + "'; known types are ['attention', 'latent_attention']");
+        }
+        Json mlp;
+        if (!l["mlp"].is_null()) {
+            const Json& f = regipel_object(l, "mlp", where);
+            const std::string fw = where + "mlp.";
+            const std::string kind = f.get_string("kind", "");
+            if (kind == "dense") {
+                mlp = Json::object().set("kind", kind).set("ff", regipel_int(f, "ff", fw));
+            } else if (kind == "moe") {
+                const Json& router = regipel_object(f, "router", fw);
+                const std::string rw = fw + "router.";
+                const long long experts = regipel_int(router, "experts", rw), top = regipel_int(router, "top", rw);
+                if (top > experts) throw ConfigError("config.json: " + rw + "'top' exceeds 'experts'");
+                if (experts > 512) throw ConfigError("config.json: " + rw + "'experts' may be at most 512");
+                long long count = 1, keep = 1;
+                if (!router["groups"].is_null()) {
+                    const Json& g = regipel_object(router, "groups", rw);
+                    count = regipel_int(g, "count", rw + "groups.");
+                    keep = regipel_int(g, "keep", rw + "groups.");
+                    if (count > 64 || experts % count || keep > count)
+                        throw ConfigError("config.json: " + rw + "'groups.count' (at most 64) must divide 'experts', and 'groups.keep' may be at most 'groups.count'");
+                    if (top > keep * (experts / count))
+                        throw ConfigError("config.json: " + rw + "the kept groups hold fewer experts than 'top'");
+                }
+                mlp = Json::object().set("kind", kind)
+                          .set("expert", Json::object().set("ff", regipel_int(regipel_object(f, "expert", fw), "ff", fw + "expert.")))
+                          .set("router", Json::object().set("experts", experts).set("top", top)
+                                             .set("scale", router["scale"].is_null() ? 1.0 : regipel_number(router, "scale", rw))
+                                             .set("groups", Json::object().set("count", count).set("keep", keep)))
+                          .set("shared", f["shared"].is_null()
+                                             ? Json()
+                                             : Json::object().set("ff", regipel_int(regipel_object(f, "shared", fw), "ff", fw + "shared.")));
+            } else {
+                throw ConfigError("config.json: " + fw + "'kind' is '" + kind + "'; known kinds are ['dense', 'moe']");
+            }
+        }
+        layers.push(Json::object().set("type", type).set("mixer", mixer).set("mlp", mlp));
+    }
+    out.set("layers", layers);
+    const long long n_layers = static_cast<long long>(layers.size());
+    if (raw["loop"].is_null()) {
+        out.set("loop", Json());
+    } else {
+        const Json& loop = regipel_object(raw, "loop", "");
+        const long long start = regipel_int(loop, "start", "loop.", 0), stop = regipel_int(loop, "stop", "loop.", 0);
+        const long long times = regipel_int(loop, "times", "loop.", 1);
+        if (start > stop || stop > n_layers)
+            throw ConfigError("config.json: 'loop' must satisfy 0 <= start <= stop <= " + std::to_string(n_layers));
+        out.set("loop", Json::object().set("start", start).set("stop", stop).set("times", times));
+    }
+    for (const char* key : {"bos_token_id", "eos_token_id"})
+        if (!raw[key].is_null()) out.set(key, raw[key]);
+    return out;
+}
+
+ModelSpec vabuzen_build_spec(const Json& c) {
+    const long long W = c["width"].as_int();
+    const double eps = c["norm"]["eps"].as_double();
+    auto norm = [&](const std::string& name) {
+        PartSpec p;
+        p.kind = "dynamic_tanh";
+        p.params = Json::object().set("width", W).set("bias", true);
+        p.tensors = {{"weight", name}, {"alpha", name + ".alpha"}, {"bias", name + ".b"}};
+        return p;
+    };
+    auto rope = [&](const Json& rot, const Json& head_dim, const char* pairing) {
+        PartSpec p;
+        p.kind = "rope";
+        p.params = Json::object().set("theta", rot["base"]).set("rotary_dim", rot["dims"]).set("head_dim", head_dim).set("pairing", pairing);
+        return p.to_json();
+    };
+    ModelSpec spec;
+    int i = 0;
+    for (const Json& l : c["layers"].items()) {
+        const std::string p = "l" + std::to_string(i) + ".";
+        const Json& m = l["mixer"];
+        LayerSpec layer;
+        layer.arrangement = "sandwich_norm";
+        layer.residual_scale = c["residual_mult"].as_double();
+        if (l["type"].as_string() == "attention") {
+            layer.mixer.kind = "biased_attention";
+            layer.mixer.params = Json::object().set("width", W).set("heads", m["heads"]).set("kv_heads", m["kv_heads"])
+                                     .set("head_dim", m["dim"]).set("v_dim", m["vdim"]).set("scale", m["scale"]).set("sink_one", true)
+                                     .set("taps", m["conv"]);
+            if (!m["mask"].is_null()) layer.mixer.params.set("window", m["mask"]["size"]).set("keep_first", m["mask"]["keep_first"]);
+            if (!m["rot"].is_null()) layer.mixer.params.set("position", rope(m["rot"], m["dim"], "neighbours"));
+            layer.mixer.tensors = {{"q", p + "mix.q"}, {"k", p + "mix.k"}, {"v", p + "mix.v"}, {"o", p + "mix.o"}};
+            if (m["conv"].as_int() > 0)
+                for (const char* t : {"q", "k", "v"}) layer.mixer.tensors.emplace_back(std::string(t) + "_conv", p + "mix." + t + ".conv");
+        } else {
+            layer.mixer.kind = "latent_attention";
+            layer.mixer.params = Json::object().set("width", W).set("heads", m["heads"]).set("dim", m["dim"])
+                                     .set("rot_dim", m["rot_dim"]).set("vdim", m["vdim"]).set("kv_rank", m["kv_rank"])
+                                     .set("scale", m["scale"]).set("eps", eps).set("sink", false).set("gate", false);
+            if (!m["rot"].is_null()) layer.mixer.params.set("position", rope(m["rot"], m["rot_dim"], "halves"));
+            layer.mixer.tensors = {{"q", p + "mix.q"},   {"dkv", p + "mix.dkv"}, {"dkv_norm", p + "mix.dkv.norm"},
+                                   {"uk", p + "mix.uk"}, {"uv", p + "mix.uv"},   {"o", p + "mix.o"}};
+        }
+        layer.mixer_norm = norm(p + "norm1");
+        layer.mixer_post_norm = norm(p + "norm1b");
+        if (l["mlp"].is_null()) {
+            layer.ffn.kind = "none";
+            layer.ffn_norm.kind = "identity";
+        } else {
+            const Json& f = l["mlp"];
+            if (f["kind"].as_string() == "dense") {
+                layer.ffn.kind = "mlp";
+                layer.ffn.params = Json::object().set("width", W).set("ff", f["ff"]).set("activation", "gelu_tanh").set("bias", true);
+                layer.ffn.tensors = {{"up", p + "mlp.up"}, {"up_bias", p + "mlp.up.b"}, {"down", p + "mlp.down"}, {"down_bias", p + "mlp.down.b"}};
+            } else {
+                const long long experts = f["router"]["experts"].as_int();
+                layer.ffn.kind = "routed_experts";
+                layer.ffn.params = Json::object().set("width", W).set("ff", f["expert"]["ff"]).set("experts", experts)
+                                       .set("top", f["router"]["top"]).set("score", "sigmoid").set("renormalize", true)
+                                       .set("renormalize_eps", 1e-20).set("route_scale", f["router"]["scale"])
+                                       .set("groups", f["router"]["groups"]).set("weight_on", "output");
+                layer.ffn.tensors = {{"router", p + "mlp.router"}};
+                for (long long e = 0; e < experts; ++e) {
+                    const std::string ep = p + "mlp.e" + std::to_string(e) + ".", n = std::to_string(e);
+                    layer.ffn.tensors.emplace_back("gate." + n, ep + "gate");
+                    layer.ffn.tensors.emplace_back("up." + n, ep + "up");
+                    layer.ffn.tensors.emplace_back("down." + n, ep + "down");
+                }
+                if (!f["shared"].is_null()) {
+                    PartSpec shared;
+                    shared.kind = "swiglu";
+                    shared.params = Json::object().set("width", W).set("ff", f["shared"]["ff"]);
+                    layer.ffn.params.set("shared", shared.to_json());
+                    for (const char* t : {"gate", "up", "down"})
+                        layer.ffn.tensors.emplace_back(std::string("shared.") + t, p + "mlp.shared." + t);
+                }
+            }
+            layer.ffn_norm = norm(p + "norm2");
+            layer.ffn_post_norm = norm(p + "norm2b");
+        }
+        spec.layers.push_back(std::move(layer));
+        ++i;
+    }
+    const int n_layers = i;
+    if (c["loop"].is_null()) {
+        for (int l = 0; l < n_layers; ++l) spec.order.push_back(RunStep{l, {}, false, 0});
+    } else {
+        const int start = static_cast<int>(c["loop"]["start"].as_int()), stop = static_cast<int>(c["loop"]["stop"].as_int());
+        const int times = static_cast<int>(c["loop"]["times"].as_int());
+        for (int l = 0; l < start; ++l) spec.order.push_back(RunStep{l, {}, false, 0});
+        for (int pass = 0; pass < times; ++pass)
+            for (int l = start; l < stop; ++l) spec.order.push_back(RunStep{l, {}, l == start, pass});
+        for (int l = stop; l < n_layers; ++l) spec.order.push_back(RunStep{l, {}, false, 0});
+        if (stop > start) {
+            // before every run: the run's own vector; from the second run on, the embedding's rows as well
+            spec.reinjection.kind = "add_rows";
+            spec.reinjection.params = Json::object().set("width", W).set("times", times).set("embedding_from", 1);
+            spec.reinjection.tensors = {{"step", "loop.step"}};
+        }
+    }
+    spec.architecture = "Vabuzen";
+    spec.vocab_size = static_cast<int>(c["vocab"].as_int());
+    spec.hidden_size = static_cast<int>(W);
+    spec.max_context = static_cast<int>(c["max_context"].as_int());
+    spec.embedding.kind = "embedding";
+    spec.embedding.params = Json::object().set("vocab", c["vocab"]).set("width", W);
+    spec.embedding.tensors = {{"table", "embed"}};
+    spec.head.kind = "linear_head";
+    spec.head.params = Json::object().set("vocab", c["vocab"]).set("width", W);
+    if (!c["logit_softcap"].is_null()) spec.head.params.set("softcap", c["logit_softcap"]);
+    spec.head.tensors = {{"weight", "head"}};
+    spec.final_norm = norm("final.norm");
+    if (c["eos_token_id"].is_array())
+        for (const Json& e : c["eos_token_id"].items()) spec.eos_token_ids.push_back(static_cast<int>(e.as_int()));
+    else if (c["eos_token_id"].is_int())
+        spec.eos_token_ids.push_back(static_cast<int>(c["eos_token_id"].as_int()));
+    if (c["bos_token_id"].is_int()) spec.bos_token_id = static_cast<int>(c["bos_token_id"].as_int());
+    spec.validate();
+    return spec;
+}
+
+}  // namespace
+
 namespace {
 void register_builtin() {
     Architecture lfm2;
@@ -1092,6 +1356,13 @@ void register_builtin() {
     kivorax.build_spec = kivorax_build_spec;
     table()["Kivorax"] = kivorax;
     table()["kivorax"] = kivorax;
+    Architecture vabuzen;
+    vabuzen.name = "Vabuzen";
+    vabuzen.aliases = {"vabuzen"};
+    vabuzen.read_config = vabuzen_read_config;
+    vabuzen.build_spec = vabuzen_build_spec;
+    table()["Vabuzen"] = vabuzen;
+    table()["vabuzen"] = vabuzen;
 }
 
 }  // namespace

@@ -55,10 +55,11 @@ int celeg_latent_attention_fast(int form, const void* q, int ldq, const void* po
                                 int ldo, float* ws_o, float* ws_ml, int n_splits, int blocks_per_split, int heads, int rank,
                                 int rot, int page_tokens, int n_layers, int layer, float scale, hipStream_t stream);
 // moe.hip
-int celeg_moe_route(const float* logits, int rows, int experts, int top, int score, int renorm, int* ids, float* weights,
-                    hipStream_t stream);
+int celeg_moe_route(const float* logits, int rows, int experts, int top, int score, int renorm, int groups, int keep,
+                    float renorm_eps, float scale, int* ids, float* weights, hipStream_t stream);
 int celeg_moe_router(const void* x, int x_dtype, const float* w, int rows, int width, int experts, int top, int score,
-                     int renorm, int* ids, float* weights, hipStream_t stream);
+                     int renorm, int groups, int keep, float renorm_eps, float scale, int* ids, float* weights,
+                     hipStream_t stream);
 int celeg_moe_tile_rows(int matrix_cores);
 int celeg_moe_plan(const int* ids, int n, int experts, int tile_rows, int* offsets, int* place_of, int* entry_at, int* tile_expert,
                    int* tile_row0, int* n_tiles, hipStream_t stream);
@@ -67,8 +68,8 @@ int celeg_moe_gather(const void* x, int dtype, const int* entry_at, const float*
 int celeg_moe_product(const void* a, const void* w, void* out, int dtype, int N, int K, int gated, int act, const int* offsets,
                       const int* tile_expert, const int* tile_row0, const int* n_tiles, int max_tiles, int tile_rows, int wide,
                       hipStream_t stream);
-int celeg_moe_combine(const void* y, int dtype, const int* place_of, const float* weights, void* out, int rows, int top,
-                      int width, hipStream_t stream);
+int celeg_moe_combine(const void* y, int dtype, const int* place_of, const float* weights, const void* base, void* out, int rows,
+                      int top, int width, hipStream_t stream);
 // gemm_f32.hip
 int celeg_gemm_f32(const float* X, int ldx, const float* W, int ldw, const float* bias, float* Y, int ldy, int M,
                    int N, int K, hipStream_t stream);
@@ -180,6 +181,14 @@ int celeg_token_gate(const void* z, int ldz, const void* table, int ld_table, in
 int celeg_normed_mean(const void* a, int lda, const float* wa, const void* b, int ldb, const float* wb, float eps, float factor,
                       void* out, int dtype, int rows, int width, hipStream_t stream);
 int celeg_depth_mix(float* history, size_t entry_stride, float* h, const float* w, int n, int rows, int width, hipStream_t stream);
+int celeg_stream_add(float* h, const float* rows, const float* vec, int n_rows, int width, hipStream_t stream);
+int celeg_softcap(float* x, size_t n, float cap, hipStream_t stream);
+// conv_rope.hip
+int celeg_conv_rope_store(const void* proj, int ld, int dtype, const float* conv_w, const float* conv_state, size_t state_stride,
+                          const int* positions, const int* token_seq, const int* seq_start, const int* token_slot,
+                          const float* inv_freq, int rotary_dim, int pairing, void* q_out, int ldq, void* k_pool, void* v_pool,
+                          const int* table, int table_stride, int n_tokens, int H, int G, int D, int V, int taps, int page_tokens,
+                          int n_layers, int layer, hipStream_t stream);
 // biased_attention.hip
 int celeg_kv_store(const void* k, int ldk, const void* v, int ldv, int dtype, void* k_pool, void* v_pool, const int* table,
                    int table_stride, const int* token_slot, const int* positions, int n_tokens, int kv_heads, int head_dim, int v_dim,
@@ -188,14 +197,14 @@ int celeg_biased_attention(const void* q, int ldq, int dtype, const void* k_pool
                            int table_stride, const int* token_slot, const int* positions, const float* r1, const float* r2,
                            const void* gate, int ldg, void* out, int ldo, int n_tokens, int q_heads, int kv_heads, int head_dim,
                            int v_dim, int page_tokens, int n_layers, int layer, float scale, float coef, int every, int window,
-                           hipStream_t stream);
+                           int keep_first, int sink_one, hipStream_t stream);
 // biased_attention_fast.hip
 int celeg_biased_attention_fast_ok(int head_dim, int v_dim);
 int celeg_biased_attention_fast(int form, const void* q, int ldq, const void* k_pool, const void* v_pool, const int* table, int table_stride,
                                 const int* cu_seqlens, const int* seq_slot, const int* seq_start, int n_seqs, int max_tiles,
                                 const float* r1, const float* r2, const void* gate, int ldg, void* out, int ldo, int q_heads,
                                 int kv_heads, int head_dim, int v_dim, int page_tokens, int n_layers, int layer, float scale, float coef,
-                                int every, int window, hipStream_t stream);
+                                int every, int window, int keep_first, int sink_one, hipStream_t stream);
 // linear_scan.hip
 int celeg_lru_gates(const void* x, int ldx, int dtype, const float* conv_w, const float* conv_b, const float* ra_t, const float* ra_b,
                     const float* ri_t, const float* ri_b, const float* lam, const float* conv_state, size_t state_stride,

@@ -218,7 +218,7 @@ Tensor Model::forward(const StepBatch& batch, Runtime& rt) {
             delta = Tensor();
             rt.stream_stat_blocks = 0;
             rt.stream_has_bf16 = false;
-            reinjection_->forward(h, x0, rt);
+            reinjection_->forward(h, x0, rt, spec.order[i].pass);
             rt.mark("reinjection");
         }
         delta = blocks_[layer]->forward(hs, delta, batch, caches_[i], rt);

@@ -298,34 +298,42 @@ static void plan_of(const Ops::RoutePlan& p, hipStream_t stream) {
                                 p.tile_expert.as<int>(), p.tile_row0.as<int>(), p.n_tiles.as<int>(), stream), "moe_plan");
 }
 
-Ops::RoutePlan Ops::moe_route(const Tensor& logits, int top, int score, bool renorm, bool matrix_cores, Workspace& ws) {
+static void check_route_rule(const Ops::RouteRule& r, long long experts, const char* who) {
+    need(r.score == 0 || r.score == 1, std::string(who) + ": score is sigmoid (0) or softmax (1)");
+    need(r.groups >= 1 && r.groups <= 64 && experts % r.groups == 0 && r.keep >= 1 && r.keep <= r.groups,
+         std::string(who) + ": up to 64 groups that divide the experts evenly, of which 1 to all are kept");
+    need(r.top <= r.keep * (experts / r.groups), std::string(who) + ": the kept groups hold fewer experts than a row uses");
+}
+
+Ops::RoutePlan Ops::moe_route(const Tensor& logits, const RouteRule& rule, bool matrix_cores, Workspace& ws) {
     dev(logits, "logits", DType::F32);
     need(logits.ndim == 2, "moe_route: logits must be [rows, experts]");
-    need(score == 0 || score == 1, "moe_route: score is sigmoid (0) or softmax (1)");
-    RoutePlan p = new_route_plan(logits.shape[0], logits.shape[1], top, matrix_cores, ws);
+    RoutePlan p = new_route_plan(logits.shape[0], logits.shape[1], rule.top, matrix_cores, ws);
+    check_route_rule(rule, p.experts, "moe_route");
     took(Path::RoutedExperts);
-    kernel_check(celeg_moe_route(logits.as<float>(), static_cast<int>(logits.shape[0]), p.experts, top, score, renorm ? 1 : 0,
-                                 p.ids.as<int>(), p.weights.as<float>(), stream), "moe_route");
+    kernel_check(celeg_moe_route(logits.as<float>(), static_cast<int>(logits.shape[0]), p.experts, rule.top, rule.score, rule.renorm ? 1 : 0,
+                                 rule.groups, rule.keep, rule.renorm_eps, rule.scale, p.ids.as<int>(), p.weights.as<float>(), stream),
+                 "moe_route");
     plan_of(p, stream);
     return p;
 }
 
-Ops::RoutePlan Ops::moe_route_rows(const Tensor& x, const Tensor& router, int top, int score, bool renorm, bool matrix_cores,
-                                   Workspace& ws) {
+Ops::RoutePlan Ops::moe_route_rows(const Tensor& x, const Tensor& router, const RouteRule& rule, bool matrix_cores, Workspace& ws) {
     dev(x, "x");
     dev(router, "router", DType::F32);
     need(x.ndim == 2 && x.contiguous() && router.ndim == 2 && router.shape[1] == x.shape[1], "moe_route_rows: x [rows, width], router [experts, width]");
-    need(score == 0 || score == 1, "moe_route_rows: score is sigmoid (0) or softmax (1)");
     const long long rows = x.shape[0], width = x.shape[1], experts = router.shape[0];
     if (!use_router_kernel || 4 * (width + experts) * 4 > 64 * 1024) {
         Tensor logits = ws.buf("moe_logits", DType::F32, {rows, experts});
         linear(x, router, logits, nullptr, ws);
-        return moe_route(logits, top, score, renorm, matrix_cores, ws);
+        return moe_route(logits, rule, matrix_cores, ws);
     }
-    RoutePlan p = new_route_plan(rows, experts, top, matrix_cores, ws);
+    RoutePlan p = new_route_plan(rows, experts, rule.top, matrix_cores, ws);
+    check_route_rule(rule, experts, "moe_route_rows");
     took(Path::RoutedExperts);
     kernel_check(celeg_moe_router(x.data, dt(x, "x"), router.as<float>(), static_cast<int>(rows), static_cast<int>(width), p.experts,
-                                  top, score, renorm ? 1 : 0, p.ids.as<int>(), p.weights.as<float>(), stream), "moe_router");
+                                  rule.top, rule.score, rule.renorm ? 1 : 0, rule.groups, rule.keep, rule.renorm_eps, rule.scale,
+                                  p.ids.as<int>(), p.weights.as<float>(), stream), "moe_router");
     plan_of(p, stream);
     return p;
 }
@@ -356,12 +364,18 @@ void Ops::moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool 
                                    p.n >= 8 * p.experts ? 1 : 0, stream), "moe_product");
 }
 
-void Ops::moe_combine(const Tensor& y, const RoutePlan& p, bool weighted, const Tensor& out) {
+void Ops::moe_combine(const Tensor& y, const RoutePlan& p, bool weighted, const Tensor& out, const Tensor* base) {
     dev(y, "y");
     dev(out, "out", y.dtype);
     need(y.ndim == 2 && out.ndim == 2 && y.shape[0] == p.n && out.shape[0] * p.top == p.n && y.shape[1] == out.shape[1],
          "moe_combine: y [rows * top, width], out [rows, width]");
-    kernel_check(celeg_moe_combine(y.data, dt(y, "y"), p.place_of.as<int>(), weighted ? p.weights.as<float>() : nullptr, out.data,
+    if (base) {
+        dev(*base, "base", y.dtype);
+        need(base->ndim == 2 && base->shape[0] == out.shape[0] && base->shape[1] == out.shape[1] && base->contiguous(),
+             "moe_combine: base must have the shape of out");
+    }
+    kernel_check(celeg_moe_combine(y.data, dt(y, "y"), p.place_of.as<int>(), weighted ? p.weights.as<float>() : nullptr,
+                                   base ? base->data : nullptr, out.data,
                                    static_cast<int>(out.shape[0]), p.top, static_cast<int>(y.shape[1]), stream), "moe_combine");
 }
 
@@ -387,7 +401,7 @@ void Ops::rmsnorm(const Tensor& x, const Tensor& weight, float eps, const Tensor
 
 // ---------------------------------------------------------------------------- norms as kernel arguments
 static CelegNorm norm_arg(const Ops::NormParams* p, long long width, const char* who) {
-    CelegNorm n{nullptr, nullptr, 0.f, CELEG_NORM_NONE};
+    CelegNorm n{nullptr, nullptr, 0.f, CELEG_NORM_NONE, 1.f, 1.f};
     if (!p) return n;
     if (p->weight.defined()) {
         dev(p->weight, "norm weight", DType::F32);
@@ -400,12 +414,13 @@ static CelegNorm norm_arg(const Ops::NormParams* p, long long width, const char*
         n.b = p->bias.as<float>();
     }
     n.eps = p->eps;
-    n.mode = p->plain ? CELEG_NORM_NONE : p->centered ? CELEG_NORM_LAYER : CELEG_NORM_RMS;
+    n.mode = p->plain ? CELEG_NORM_NONE : p->tanh ? CELEG_NORM_TANH : p->centered ? CELEG_NORM_LAYER : CELEG_NORM_RMS;
+    n.alpha = p->alpha;
     return n;
 }
 
 void Ops::norm_step(const Tensor& h, const Tensor* y, const NormParams* post, const NormParams* pre, const Tensor* out,
-                    const int* rows) {
+                    const int* rows, float gain) {
     dev(h, "h", DType::F32);
     need(h.ndim == 2, "norm_step: h must be a matrix");
     const long long width = h.shape[1];
@@ -424,7 +439,9 @@ void Ops::norm_step(const Tensor& h, const Tensor* y, const NormParams* post, co
     }
     need(!rows || out, "norm_step: a list of rows goes with an output");
     need(y || out, "norm_step: nothing to do");
-    kernel_check(celeg_norm_step(h.as<float>(), y ? y->data : nullptr, y ? dt(*y, "y") : 0, norm_arg(y ? post : nullptr, width, "norm_step"),
+    CelegNorm post_arg = norm_arg(y ? post : nullptr, width, "norm_step");
+    post_arg.gain = gain;
+    kernel_check(celeg_norm_step(h.as<float>(), y ? y->data : nullptr, y ? dt(*y, "y") : 0, post_arg,
                                  norm_arg(pre, width, "norm_step"), out ? out->data : nullptr, out ? dt(*out, "out") : 0, rows,
                                  static_cast<int>(n_rows), static_cast<int>(width), y && !rows ? 1 : 0, stream), "norm_step");
 }
@@ -1024,7 +1041,8 @@ void Ops::biased_attention(const Tensor& q, const Tensor& out, const ScoreShape&
         dev(*r2, "r2", DType::F32);
         need(r1->numel() == s.heads && r2->numel() == s.heads, "biased_attention: one pair of bias numbers per head");
     }
-    need(s.every >= 0 && s.window >= 0, "biased_attention: every and window are not negative");
+    need(s.every >= 0 && s.window >= 0 && s.keep_first >= 0, "biased_attention: every, window and keep_first are not negative");
+    const int keep_first = s.window > 0 ? s.keep_first : 0, sink_one = s.sink_one ? 1 : 0;
     if (gate) {
         dev(*gate, "gate", q.dtype, false);
         need(gate->ndim == 2 && gate->shape[0] == T && gate->shape[1] == out.shape[1], "biased_attention: gate [rows, heads * v_dim]");
@@ -1046,14 +1064,76 @@ void Ops::biased_attention(const Tensor& q, const Tensor& out, const ScoreShape&
                                                  batch.seq_start, batch.n_seqs, max_tiles, r1 ? r1->as<float>() : nullptr,
                                                  r2 ? r2->as<float>() : nullptr, gate ? gate->data : nullptr, ldg, out.data, ldo, s.heads,
                                                  s.kv_heads, s.head_dim, s.v_dim, kv.page_tokens, kv.n_layers, kv.layer, s.scale, s.coef,
-                                                 s.every, s.window, stream), "biased attention (bfloat16, matrix cores)");
+                                                 s.every, s.window, keep_first, sink_one, stream), "biased attention (bfloat16, matrix cores)");
         return;
     }
     kernel_check(celeg_biased_attention(q.data, rows_of(q, "q"), dt(q, "q"), kv.k, kv.v, kv.table, kv.table_stride, batch.token_slot,
                                         batch.positions, r1 ? r1->as<float>() : nullptr, r2 ? r2->as<float>() : nullptr,
                                         gate ? gate->data : nullptr, gate ? rows_of(*gate, "gate") : 0, out.data, rows_of(out, "out"),
                                         static_cast<int>(T), s.heads, s.kv_heads, s.head_dim, s.v_dim, kv.page_tokens, kv.n_layers,
-                                        kv.layer, s.scale, s.coef, s.every, s.window, stream), "biased_attention");
+                                        kv.layer, s.scale, s.coef, s.every, s.window, keep_first, sink_one, stream), "biased_attention");
+}
+
+void Ops::conv_rope_store(const Tensor& proj, const Tensor* conv_w, const Tensor* conv_state, int taps, const Tensor* inv_freq,
+                          int rotary_dim, int pairing, const Tensor& q_out, int heads, const StepBatch& batch, const KVView& kv) {
+    dev(proj, "proj");
+    dev(q_out, "q_out", proj.dtype, false);
+    check_kv_wide(kv, kv.kv_heads, kv.head_dim, kv.v_head_dim, proj.dtype, "conv_rope_store");
+    const long long T = batch.n_tokens, D = kv.head_dim, V = kv.v_head_dim, G = kv.kv_heads;
+    const long long channels = (heads + G) * D + G * V;
+    need(heads > 0 && proj.ndim == 2 && proj.shape[0] == T && proj.shape[1] >= channels, "conv_rope_store: proj holds q | k | v of every row");
+    need(q_out.ndim == 2 && q_out.shape[0] == T && q_out.shape[1] == heads * D, "conv_rope_store: q_out [rows, heads * head_dim]");
+    need((conv_w == nullptr) == (conv_state == nullptr), "conv_rope_store: taps and saved inputs go together");
+    need(std::max(D, V) * 4 <= 60 * 1024, "conv_rope_store: heads of more than 15,360 values are not supported");
+    if (conv_w) {
+        dev(*conv_w, "conv_w", DType::F32);
+        dev(*conv_state, "conv_state", DType::F32, false);
+        need(taps >= 1 && conv_w->ndim == 2 && conv_w->shape[0] == channels && conv_w->shape[1] == taps,
+             "conv_rope_store: conv_w must be [channels, taps]");
+        need(conv_state->ndim == 3 && conv_state->shape[1] == std::max(taps - 1, 1) && conv_state->shape[2] == channels &&
+                 conv_state->stride[2] == 1 && conv_state->stride[1] == channels,
+             "conv_rope_store: the saved inputs must be [slots, taps - 1, channels]");
+    } else {
+        taps = 1;
+    }
+    if (inv_freq) {
+        dev(*inv_freq, "inv_freq", DType::F32);
+        need(rotary_dim > 0 && rotary_dim % 2 == 0 && rotary_dim <= D && inv_freq->numel() == rotary_dim / 2 && (pairing == 0 || pairing == 1),
+             "conv_rope_store: an even number of turned values, at most a head's, with a frequency a pair");
+    }
+    const size_t state_stride = conv_state ? static_cast<size_t>(conv_state->stride[0]) : 0;
+    kernel_check(celeg_conv_rope_store(proj.data, rows_of(proj, "proj"), dt(proj, "proj"), conv_w ? conv_w->as<float>() : nullptr,
+                                       conv_state ? conv_state->as<float>() : nullptr, state_stride, batch.positions, batch.token_seq,
+                                       batch.seq_start, batch.token_slot, inv_freq ? inv_freq->as<float>() : nullptr,
+                                       inv_freq ? rotary_dim : 0, pairing, q_out.data, rows_of(q_out, "q_out"), kv.k, kv.v, kv.table,
+                                       kv.table_stride, static_cast<int>(T), heads, static_cast<int>(G), static_cast<int>(D),
+                                       static_cast<int>(V), taps, kv.page_tokens, kv.n_layers, kv.layer, stream), "conv_rope_store");
+    // (after every row has read the old saved inputs)
+    if (conv_w && taps > 1)
+        kernel_check(celeg_delta_conv_state(proj.data, rows_of(proj, "proj"), dt(proj, "proj"), conv_state->as<float>(), state_stride,
+                                            batch.cu_seqlens, batch.seq_slot, batch.n_seqs, static_cast<int>(channels), taps, stream),
+                     "conv_rope_store (saved inputs)");
+}
+
+void Ops::stream_add(const Tensor& h, const Tensor* rows_in, const Tensor* vec) {
+    dev(h, "h", DType::F32);
+    need(h.ndim == 2, "stream_add: h must be a matrix");
+    if (rows_in) {
+        dev(*rows_in, "rows", DType::F32);
+        need(rows_in->ndim == 2 && rows_in->shape[0] == h.shape[0] && rows_in->shape[1] == h.shape[1], "stream_add: rows must have the shape of h");
+    }
+    if (vec) {
+        dev(*vec, "vec", DType::F32);
+        need(vec->numel() == h.shape[1], "stream_add: the vector must have the width of h");
+    }
+    kernel_check(celeg_stream_add(h.as<float>(), rows_in ? rows_in->as<float>() : nullptr, vec ? vec->as<float>() : nullptr,
+                                  static_cast<int>(h.shape[0]), static_cast<int>(h.shape[1]), stream), "stream_add");
+}
+
+void Ops::softcap(const Tensor& x, float cap) {
+    dev(x, "x", DType::F32);
+    need(cap > 0.f, "softcap: the cap must be positive");
+    kernel_check(celeg_softcap(x.as<float>(), static_cast<size_t>(x.numel()), cap, stream), "softcap");
 }
 
 // ---------------------------------------------------------------------------- layer glue

@@ -157,16 +157,21 @@ public:
     // What a norm does to a row, for kernels that take a norm as an argument: weight and bias
     // (32-bit, either may be undefined), eps, and whether the mean is taken off first (a layer
     // norm) or not (an RMS norm); `plain`: no normalisation at all.
+    // `tanh`: no statistics at all, every value becomes tanh(alpha * x) before weight and bias.
     struct NormParams {
         Tensor weight, bias;
-        float eps = 0.f;
-        bool centered = false, plain = false;
+        float eps = 0.f, alpha = 1.f;
+        bool centered = false, plain = false, tanh = false;
     };
     // One sub-layer boundary on a single 32-bit stream h [rows, width]: if y is given,
-    // h += post(y) (post null: the plain sum); then, if out is given, out = pre(h).  With `rows`
+    // h += gain * post(y) (post null: the plain sum); then, if out is given, out = pre(h).  With `rows`
     // only those rows of h are read, nothing is written back, and out has one row per entry.
     void norm_step(const Tensor& h, const Tensor* y, const NormParams* post, const NormParams* pre, const Tensor* out,
-                   const int* rows = nullptr);
+                   const int* rows = nullptr, float gain = 1.0f);
+    // h [rows, width] += (rows_in [rows, width] +) vec [width], all 32-bit; either addend may be null
+    void stream_add(const Tensor& h, const Tensor* rows_in, const Tensor* vec);
+    // x <- cap * tanh(x / cap), 32-bit x
+    void softcap(const Tensor& x, float cap);
     // out [rows, 2 * width] = (a | b), both 32-bit [rows, width]
     void concat_rows(const Tensor& a, const Tensor& b, const Tensor& out);
     void swiglu(const Tensor& gate_up, const Tensor& out);
@@ -233,7 +238,21 @@ public:
     // Softmax attention whose positions enter through the scores: score = (q . k) * scale * f(i) - r1[h] ln(1 + r2[h] (i - j)),
     // f(i) = 1 + coef ln(floor((i + 1) / every) + 1) (every 0: f = 1); r1, r2 [heads] 32-bit or null.  Values of kv.v_head_dim.
     // gate: raw values [rows, heads * v_dim] (a view with dense rows) whose sigmoid multiplies the result, or null.
-    struct ScoreShape { int heads = 0, kv_heads = 0, head_dim = 0, v_dim = 0, window = 0, every = 0; float scale = 1.f, coef = 0.f; };
+    // With a window, `keep_first` keys at the start of the sequence stay visible however far the window has moved;
+    // `sink_one`: the softmax's denominator holds a one more (a key of score 0 that has no value).
+    struct ScoreShape {
+        int heads = 0, kv_heads = 0, head_dim = 0, v_dim = 0, window = 0, every = 0;
+        float scale = 1.f, coef = 0.f;
+        int keep_first = 0;
+        bool sink_one = false;
+    };
+    // What lies between an attention's q/k/v product and its scores where the projected channels pass a short causal
+    // convolution: proj [rows, >= (heads + kv_heads) * head_dim + kv_heads * v_dim] holds q | k | v from column 0;
+    // conv_w [channels, taps] 32-bit continues from conv_state [slots, taps - 1, channels] 32-bit (both null: no
+    // convolution), which is moved on afterwards; q and k heads turn by the rows' positions (inv_freq null: not);
+    // the queries go to q_out [rows, heads * head_dim], keys and values to the rows' places in the pages.
+    void conv_rope_store(const Tensor& proj, const Tensor* conv_w, const Tensor* conv_state, int taps, const Tensor* inv_freq,
+                         int rotary_dim, int pairing, const Tensor& q_out, int heads, const StepBatch& batch, const KVView& kv);
     // a step's keys [rows, kv_heads * head_dim] and values [rows, kv_heads * v_dim] to their places in the pages
     void kv_store(const Tensor& k, const Tensor& v, const StepBatch& batch, const KVView& kv);
     void biased_attention(const Tensor& q, const Tensor& out, const ScoreShape& shape, const Tensor* r1, const Tensor* r2,
@@ -276,13 +295,22 @@ public:
         Tensor tile_expert, tile_row0, n_tiles;
         int n = 0, top = 0, experts = 0, max_tiles = 0, tile_rows = 0;
     };
-    // logits [rows, experts] 32-bit -> the plan; score "sigmoid" (0) or "softmax" (1); matrix_cores: the
-    // plan's products all run on the matrix cores (moe_matrix_cores_ok for each of them)
-    RoutePlan moe_route(const Tensor& logits, int top, int score, bool renorm, bool matrix_cores, Workspace& ws);
+    // How a row's experts are chosen and weighted: score "sigmoid" (0) or "softmax" (1); with groups > 1 the experts
+    // form that many equal runs of neighbours, a run's score is the sum of its two largest scores, and only the experts
+    // of the `keep` best runs can be chosen; the `top` largest scores are the weights, with `renorm` divided by their
+    // sum plus renorm_eps, then times `scale`.
+    struct RouteRule {
+        int top = 1, score = 0;
+        bool renorm = false;
+        float renorm_eps = 0.f, scale = 1.f;
+        int groups = 1, keep = 1;
+    };
+    // logits [rows, experts] 32-bit -> the plan; matrix_cores: the plan's products all run on the matrix cores
+    // (moe_matrix_cores_ok for each of them)
+    RoutePlan moe_route(const Tensor& logits, const RouteRule& rule, bool matrix_cores, Workspace& ws);
     // the same from the rows themselves: x [rows, width] times the router's 32-bit matrix [experts, width],
     // the product in 32-bit inside the routing kernel
-    RoutePlan moe_route_rows(const Tensor& x, const Tensor& router, int top, int score, bool renorm, bool matrix_cores,
-                             Workspace& ws);
+    RoutePlan moe_route_rows(const Tensor& x, const Tensor& router, const RouteRule& rule, bool matrix_cores, Workspace& ws);
     // whether a product of experts [.., N, K] in this dtype runs on the matrix cores
     bool moe_matrix_cores_ok(DType dtype, long long N, long long K) const {
         return use_moe_mfma && dtype == DType::BF16 && K % 32 == 0 && N % 16 == 0;
@@ -291,7 +319,8 @@ public:
     // out[p] = a[p] w[expert of p]^T; w [experts * N, K], or [experts * 2N, K] if gated (silu(gate) * up)
     // (not gated, act 1: the square of relu of the product)
     void moe_product(const Tensor& a, const Tensor& w, const Tensor& out, bool gated, const RoutePlan& plan, int act = 0);
-    void moe_combine(const Tensor& y, const RoutePlan& plan, bool weighted, const Tensor& out);
+    // base: rows [rows, width] added to every row's sum (what all rows get besides their experts), or null
+    void moe_combine(const Tensor& y, const RoutePlan& plan, bool weighted, const Tensor& out, const Tensor* base = nullptr);
     // sampling
     void sample(const Tensor& logits, const float* fparams, const int* iparams, uint8_t* seen,
                 size_t seen_stride, int* out_tokens, int* last_tokens, bool all_greedy, Workspace& ws,

@@ -715,6 +715,10 @@ private:
 // ("renormalize": divided by their sum).  "weight_on": "input" (the output is
 // sum expert(w x)) or "output" (sum w expert(x)).  "gated": false makes an expert
 // W_down act(W_up x) with "activation": "relu2" (the square of relu) and no gate matrix.
+// "groups": {"count", "keep"}: the experts form `count` equal groups of neighbours, a group's score is the
+// sum of its two largest scores, and only experts of the `keep` best groups can be chosen.  "renormalize_eps"
+// is added to the sum the chosen scores are divided by; "route_scale" multiplies the weights afterwards.
+// "shared": a feed-forward part that every row passes as well; its output is added to the experts'.
 class RoutedExperts final : public FeedForward {
 public:
     explicit RoutedExperts(const PartSpec& s) : FeedForward(s) {
@@ -728,15 +732,30 @@ public:
         if (on != "input" && on != "output") throw SpecError("routed_experts: weight_on is 'input' or 'output', not '" + on + "'");
         score_ = score == "softmax" ? 1 : 0;
         on_input_ = on == "input";
-        renorm_ = p.get_bool("renormalize", false);
+        rule_.renorm = p.get_bool("renormalize", false);
+        rule_.renorm_eps = static_cast<float>(p.get_double("renormalize_eps", 0.0));
+        rule_.scale = static_cast<float>(p.get_double("route_scale", 1.0));
+        if (!p["groups"].is_null()) {
+            rule_.groups = static_cast<int>(p["groups"].get_int("count", 1));
+            rule_.keep = static_cast<int>(p["groups"].get_int("keep", rule_.groups));
+        }
+        if (PartSpec::is_part(p["shared"])) shared_ = build_as<FeedForward>("ffn", PartSpec::from_json(p["shared"], "routed_experts.shared"));
         gated_ = p.get_bool("gated", true);
         const std::string act = p.get_string("activation", gated_ ? "silu" : "relu2");
         if (act != (gated_ ? "silu" : "relu2"))
             throw SpecError("routed_experts: activation is 'silu' for gated experts and 'relu2' for experts without a gate, not '" + act + "'");
         if (width_ <= 0 || ff_ <= 0 || experts_ <= 0 || top_ <= 0 || top_ > experts_)
             throw SpecError("routed_experts: width, ff and experts must be positive and top between 1 and experts");
+        if (rule_.groups < 1 || rule_.groups > 64 || experts_ % rule_.groups || rule_.keep < 1 || rule_.keep > rule_.groups ||
+            top_ > rule_.keep * (experts_ / rule_.groups))
+            throw SpecError("routed_experts: groups.count (up to 64) must divide experts, and the groups.keep kept groups must hold at least top experts");
+        rule_.top = top_;
+        rule_.score = score_;
     }
-    bool graph_safe() const override { return true; }
+    bool graph_safe() const override { return !shared_ || shared_->graph_safe(); }
+    std::vector<const Part*> children() const override {
+        return shared_ ? std::vector<const Part*>{shared_.get()} : std::vector<const Part*>{};
+    }
     static std::string role(const char* what, int e) { return std::string(what) + "." + std::to_string(e); }
     WeightSpecs weight_specs() const override {
         WeightSpecs specs{{"router", WeightSpec{{experts_, width_}, "vector", "normal", {}}}};
@@ -745,10 +764,18 @@ public:
             specs.push_back({role("up", e), matrix(ff_, width_)});
             specs.push_back({role("down", e), matrix(width_, ff_)});
         }
+        // the shared part's tensors travel under "shared.<its role>"; its checkpoint names are in this part's tensor map
+        if (shared_)
+            for (const auto& ws : shared_->weight_specs()) specs.push_back({"shared." + ws.first, ws.second});
         return specs;
     }
-    void load(const PartTensors& t, Runtime&) override {
+    void load(const PartTensors& t, Runtime& rt) override {
         router_ = get(t, "router");
+        if (shared_) {
+            PartTensors mine;
+            for (const auto& ws : shared_->weight_specs()) mine[ws.first] = get(t, "shared." + ws.first);
+            shared_->load(mine, rt);
+        }
         std::vector<std::shared_ptr<DeviceTensor>> in, out;
         for (int e = 0; e < experts_; ++e) {
             if (gated_) in.push_back(get(t, role("gate", e)));
@@ -760,26 +787,32 @@ public:
         w_gate_up_ = concat_rows(in);       // [experts * 2 ff, width]: per expert its gate rows, then its up rows (no gate: [experts * ff, width])
         w_down_ = concat_rows(out);         // [experts * width, ff]
     }
-    Tensor forward(const Tensor& x, const StepBatch&, Runtime& rt) override {
+    Tensor forward(const Tensor& x, const StepBatch& batch, Runtime& rt) override {
         const long long T = x.shape[0];
+        // what every row gets besides its experts (good until the shared part's next call: this part's own
+        // result then goes to a buffer of another name than a feed-forward's usual one)
+        Tensor base;
+        if (shared_) base = shared_->forward(x, batch, rt);
         const bool cores = rt.ops.moe_matrix_cores_ok(x.dtype, ff_, width_) && rt.ops.moe_matrix_cores_ok(x.dtype, width_, ff_) &&
                            w_gate_up_->view.dtype == x.dtype;
-        const Ops::RoutePlan plan = rt.ops.moe_route_rows(x, router_->view, top_, score_, renorm_, cores, rt.ws);
+        const Ops::RoutePlan plan = rt.ops.moe_route_rows(x, router_->view, rule_, cores, rt.ws);
         Tensor a = rt.ws.buf("moe_in", rt.dtype, {T * top_, width_});
         rt.ops.moe_gather(x, plan, on_input_, a);
         Tensor act = rt.ws.buf("moe_act", rt.dtype, {T * top_, ff_});
         rt.ops.moe_product(a, w_gate_up_->view, act, gated_, plan, gated_ ? 0 : 1);
         Tensor y = rt.ws.buf("moe_y", rt.dtype, {T * top_, width_});
         rt.ops.moe_product(act, w_down_->view, y, false, plan);
-        Tensor out = rt.ws.buf("ffn_out", rt.dtype, {T, width_});
-        rt.ops.moe_combine(y, plan, !on_input_, out);
+        Tensor out = rt.ws.buf(shared_ ? "moe_out" : "ffn_out", rt.dtype, {T, width_});
+        rt.ops.moe_combine(y, plan, !on_input_, out, shared_ ? &base : nullptr);
         return out;
     }
 
 private:
     long long width_ = 0, ff_ = 0;
     int experts_ = 0, top_ = 0, score_ = 0;
-    bool on_input_ = false, renorm_ = false, gated_ = true;
+    bool on_input_ = false, gated_ = true;
+    Ops::RouteRule rule_;
+    std::unique_ptr<FeedForward> shared_;
     std::shared_ptr<DeviceTensor> router_, w_gate_up_, w_down_;
 };
 
@@ -797,7 +830,8 @@ public:
 // logits = x E_out^T with E_out = E when the head is tied, else lm_head
 // (src/backend/cpu/model_forward_token.cpp:213-218; src/model/inference/layer_bindings.cpp:24-95).
 // Logits leave in 32-bit.  "scale" on the embedding multiplies the gathered rows (in 32-bit, as
-// they enter the residual stream); "scale" on a head multiplies the logits.
+// they enter the residual stream); "scale" on a head multiplies the logits; "softcap" c > 0 bends them
+// afterwards to c * tanh(logit / c).
 class TokenEmbedding final : public Embedding {
 public:
     explicit TokenEmbedding(const PartSpec& s)
@@ -882,16 +916,18 @@ bool head_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& ba
 class TiedHead final : public Head {
 public:
     explicit TiedHead(const PartSpec& s)
-        : Head(s), vocab_(static_cast<int>(s.params.get_int("vocab", 0))), scale_(static_cast<float>(s.params.get_double("scale", 1.0))) {}
+        : Head(s), vocab_(static_cast<int>(s.params.get_int("vocab", 0))), scale_(static_cast<float>(s.params.get_double("scale", 1.0))),
+          softcap_(static_cast<float>(s.params.get_double("softcap", 0.0))) {}
     bool graph_safe() const override { return true; }
     int vocab() const override { return vocab_; }
     void forward(const Tensor& x, const Tensor& out, Runtime& rt, const Embedding* embedding) override {
         rt.ops.linear(x, table_of(embedding), out, nullptr, rt.ws);
         if (scale_ != 1.0f) rt.ops.scale(out, scale_);
+        if (softcap_ > 0.f) rt.ops.softcap(out, softcap_);
     }
     bool forward_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& batch, const Tensor& out, Runtime& rt,
                        const Embedding* embedding) override {
-        if (scale_ != 1.0f) return false;       // (what the fused head leaves beside the logits knows no scale)
+        if (scale_ != 1.0f || softcap_ > 0.f) return false;       // (what the fused head leaves beside the logits knows no scale)
         return head_fused(h, norm, batch, out, rt, table_of(embedding));
     }
 
@@ -902,14 +938,14 @@ private:
         return t;
     }
     int vocab_;
-    float scale_;
+    float scale_, softcap_;
 };
 
 class LinearHead final : public Head {
 public:
     explicit LinearHead(const PartSpec& s)
         : Head(s), vocab_(static_cast<int>(s.params.get_int("vocab", 0))), width_(s.params.get_int("width", 0)),
-          scale_(static_cast<float>(s.params.get_double("scale", 1.0))) {}
+          scale_(static_cast<float>(s.params.get_double("scale", 1.0))), softcap_(static_cast<float>(s.params.get_double("softcap", 0.0))) {}
     bool graph_safe() const override { return true; }
     int vocab() const override { return vocab_; }
     WeightSpecs weight_specs() const override { return {{"weight", matrix(vocab_, width_)}}; }
@@ -917,17 +953,18 @@ public:
     void forward(const Tensor& x, const Tensor& out, Runtime& rt, const Embedding*) override {
         rt.ops.linear(x, weight_->view, out, nullptr, rt.ws);
         if (scale_ != 1.0f) rt.ops.scale(out, scale_);
+        if (softcap_ > 0.f) rt.ops.softcap(out, softcap_);
     }
     bool forward_fused(const Tensor& h, const Norm::Foldable& norm, const StepBatch& batch, const Tensor& out, Runtime& rt,
                        const Embedding*) override {
-        if (scale_ != 1.0f) return false;
+        if (scale_ != 1.0f || softcap_ > 0.f) return false;
         return head_fused(h, norm, batch, out, rt, weight_->view);
     }
 
 private:
     int vocab_;
     long long width_;
-    float scale_;
+    float scale_, softcap_;
     std::shared_ptr<DeviceTensor> weight_;
 };
 
@@ -1123,6 +1160,43 @@ public:
 private:
     long long width_;
     double eps_;
+    bool bias_;
+    std::shared_ptr<DeviceTensor> weight_, b_;
+    Ops::NormParams params_;
+};
+
+// ---------------------------------------------------------------------------- dynamic tanh
+// y = tanh(alpha * x) * w + b: a "norm" without any statistic of the row; alpha is one learned number
+// stored beside the weight.  32-bit whatever the activation dtype.  "bias": false leaves b out.
+class DynamicTanh final : public Norm {
+public:
+    explicit DynamicTanh(const PartSpec& s) : Norm(s), width_(s.params.get_int("width", 0)), bias_(s.params.get_bool("bias", true)) {
+        if (width_ <= 0) throw SpecError("dynamic_tanh: width must be positive");
+    }
+    bool graph_safe() const override { return true; }
+    WeightSpecs weight_specs() const override {
+        WeightSpecs specs{{"weight", vec(width_, "around_one")}, {"alpha", WeightSpec{{}, "vector", "around_one", {{1}}}}};
+        if (bias_) specs.push_back({"bias", vec(width_)});
+        return specs;
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        weight_ = get(t, "weight");
+        if (bias_) b_ = get(t, "bias");
+        const std::vector<float> alpha = to_host_floats(get(t, "alpha")->view);
+        if (alpha.size() != 1) throw SpecError("dynamic_tanh: alpha is one number");
+        params_.weight = weight_->view;
+        if (b_) params_.bias = b_->view;
+        params_.alpha = alpha[0];
+        params_.tanh = true;
+    }
+    void forward(const Tensor& x, const Tensor& out, Runtime& rt, const Tensor* delta, const int* rows) override {
+        if (x.dtype != DType::F32) throw SpecError("dynamic_tanh: the rows to norm must be 32-bit");
+        rt.ops.norm_step(x, delta, nullptr, &params_, &out, rows);
+    }
+    const Ops::NormParams* params() const override { return weight_ ? &params_ : nullptr; }
+
+private:
+    long long width_;
     bool bias_;
     std::shared_ptr<DeviceTensor> weight_, b_;
     Ops::NormParams params_;
@@ -1432,7 +1506,7 @@ public:
     bool graph_safe() const override { return true; }
     WeightSpecs weight_specs() const override { return {{"weight", matrix(width_, 2 * width_)}}; }
     void load(const PartTensors& t, Runtime&) override { weight_ = get(t, "weight"); }
-    void forward(const Tensor& h, const Tensor& x0, Runtime& rt) override {
+    void forward(const Tensor& h, const Tensor& x0, Runtime& rt, int) override {
         const long long T = h.shape[0];
         Tensor both = rt.ws.buf("reinjection_in", rt.dtype, {T, 2 * width_});
         rt.ops.concat_rows(h, x0, both);
@@ -1444,16 +1518,48 @@ private:
     std::shared_ptr<DeviceTensor> weight_;
 };
 
+// add_rows: before run t of the looped range, h <- h + (x0 if t >= "embedding_from") + step[t]; step
+// [times, width] holds a learned vector per run ("steps": false: no such tensor).  All 32-bit.
+class AdditiveReinjection final : public Reinjection {
+public:
+    explicit AdditiveReinjection(const PartSpec& s)
+        : Reinjection(s), width_(s.params.get_int("width", 0)), times_(s.params.get_int("times", 1)),
+          from_(s.params.get_int("embedding_from", 1)), steps_(s.params.get_bool("steps", true)) {
+        if (width_ <= 0 || times_ <= 0 || from_ < 0) throw SpecError("add_rows: width and times must be positive, embedding_from not negative");
+    }
+    bool graph_safe() const override { return true; }
+    WeightSpecs weight_specs() const override {
+        if (!steps_) return {};
+        return {{"step", WeightSpec{{times_, width_}, "vector", "normal", {}}}};
+    }
+    void load(const PartTensors& t, Runtime&) override {
+        if (steps_) step_ = get(t, "step");
+    }
+    void forward(const Tensor& h, const Tensor& x0, Runtime& rt, int pass) override {
+        if (pass < 0 || pass >= times_) throw SpecError("add_rows: run " + std::to_string(pass) + " of " + std::to_string(times_));
+        Tensor vec;
+        if (steps_) vec = Tensor::make(step_->view.as<float>() + static_cast<size_t>(pass) * static_cast<size_t>(width_), DType::F32, {width_});
+        rt.ops.stream_add(h, pass >= from_ ? &x0 : nullptr, steps_ ? &vec : nullptr);
+    }
+
+private:
+    long long width_, times_, from_;
+    bool steps_;
+    std::shared_ptr<DeviceTensor> step_;
+};
+
 // ---------------------------------------------------------------------------- norms before and after
 // sandwich_norm: h += post1(mixer(pre1(h))); h += post2(ffn(pre2(h))).  The stream is 32-bit
 // and so are the norms' statistics and the sums.  One kernel per boundary: the first norms the
 // stream, the second adds the mixer's normed output and norms for the feed-forward, the third
 // adds the feed-forward's normed output.  A feed-forward of kind "none" is left out with its norms.
+// The layer's "residual_scale" m makes the sums h += m * post(...).
 class SandwichBlock final : public Block {
 public:
     explicit SandwichBlock(const LayerSpec& layer)
         : mixer_norm_(build_as<Norm>("norm", layer.mixer_norm)), mixer_(build_as<Mixer>("mixer", layer.mixer)),
-          mixer_post_(build_as<Norm>("norm", layer.mixer_post_norm)), has_ffn_(layer.ffn.kind != "none") {
+          mixer_post_(build_as<Norm>("norm", layer.mixer_post_norm)), has_ffn_(layer.ffn.kind != "none"),
+          gain_(static_cast<float>(layer.residual_scale)) {
         if (has_ffn_) {
             ffn_norm_ = build_as<Norm>("norm", layer.ffn_norm);
             ffn_ = build_as<FeedForward>("ffn", layer.ffn);
@@ -1479,12 +1585,12 @@ public:
         Tensor y = mixer_->forward(normed, batch, cache, rt);
         rt.mark("mixer " + mixer_->spec.kind);
         if (!has_ffn_) {
-            rt.ops.norm_step(h, &y, &of(*mixer_post_), nullptr, nullptr);
+            rt.ops.norm_step(h, &y, &of(*mixer_post_), nullptr, nullptr, nullptr, gain_);
             return Tensor();
         }
-        rt.ops.norm_step(h, &y, &of(*mixer_post_), &of(*ffn_norm_), &normed);
+        rt.ops.norm_step(h, &y, &of(*mixer_post_), &of(*ffn_norm_), &normed, nullptr, gain_);
         y = ffn_->forward(normed, batch, rt);
-        rt.ops.norm_step(h, &y, &of(*ffn_post_), nullptr, nullptr);
+        rt.ops.norm_step(h, &y, &of(*ffn_post_), nullptr, nullptr, nullptr, gain_);
         rt.mark("ffn " + ffn_->spec.kind);
         return Tensor();
     }
@@ -1499,6 +1605,7 @@ private:
     std::unique_ptr<Mixer> mixer_;
     std::unique_ptr<Norm> mixer_post_;
     bool has_ffn_;
+    float gain_ = 1.f;
     std::unique_ptr<Norm> ffn_norm_;
     std::unique_ptr<FeedForward> ffn_;
     std::unique_ptr<Norm> ffn_post_;
@@ -1511,7 +1618,13 @@ private:
 // score(i, j) = (q_i . k_j) * scale * f(i) - r1[h] ln(1 + r2[h] (i - j)) with
 // f(i) = 1 + coef ln(floor((i + 1) / every) + 1) ("query_temperature": {"coef", "every"}; absent: f = 1) and,
 // with "distance_bias", a learned pair (r1, r2) per query head.  Keys j <= i (inside "window" where one is
-// given).  "gate": "sigmoid" multiplies the heads, side by side, element by element with sigmoid(W_g h).
+// given; with "keep_first" n the first n positions of the sequence stay visible behind the window, at their
+// true positions).  "gate": "sigmoid" multiplies the heads, side by side, element by element with sigmoid(W_g h).
+// "sink_one": the softmax's denominator holds a one more, p_j = exp(s_j) / (1 + sum exp(s_j)).
+// "taps" n > 0: every channel of q, k and v passes a causal convolution over time of n taps right behind its
+// projection (tensors q_conv, k_conv, v_conv [channels, taps], no bias; y_t = sum_j w[:, j] u_(t - n + 1 + j),
+// zeros before the sequence starts); the last n - 1 projected rows are the request's state.  "position": a
+// position encoding part (rope) that turns q and k heads behind the convolution.
 class BiasedAttention final : public Mixer {
 public:
     explicit BiasedAttention(const PartSpec& s) : Mixer(s) {
@@ -1536,16 +1649,34 @@ public:
             shape_.every = static_cast<int>(t.get_int("every", 0));
             if (shape_.every <= 0) throw SpecError("biased_attention: query_temperature.every must be positive");
         }
+        if (!p["keep_first"].is_null()) {
+            shape_.keep_first = static_cast<int>(p["keep_first"].as_int());
+            if (shape_.keep_first < 0) throw SpecError("biased_attention: keep_first is not negative");
+            if (shape_.window <= 0) shape_.keep_first = 0;       // (without a window every key is visible anyway)
+        }
+        shape_.sink_one = p.get_bool("sink_one", false);
+        taps_ = static_cast<int>(p.get_int("taps", 0));
+        if (taps_ < 0) throw SpecError("biased_attention: taps is not negative");
+        if (PartSpec::is_part(p["position"]))
+            position_ = build_as<PositionEncoding>("position", PartSpec::from_json(p["position"], "biased_attention.position"));
         distance_bias_ = p.get_bool("distance_bias", false);
         const std::string gate = p.get_string("gate", "none");
         if (gate != "none" && gate != "sigmoid") throw SpecError("biased_attention: gate is 'none' or 'sigmoid', not '" + gate + "'");
         gated_ = gate == "sigmoid";
     }
     bool graph_safe() const override { return true; }
+    std::vector<const Part*> children() const override {
+        return position_ ? std::vector<const Part*>{position_.get()} : std::vector<const Part*>{};
+    }
     std::optional<KVNeed> kv_need() const override {
         KVNeed need{shape_.kv_heads, shape_.head_dim, shape_.window > 0 ? std::optional<int>(shape_.window) : std::nullopt};
         need.v_head_dim = shape_.v_dim;
+        need.keep_first = shape_.keep_first;
         return need;
+    }
+    std::vector<StateNeed> state_needs() const override {
+        if (taps_ <= 0) return {};
+        return {StateNeed{"conv", {std::max(taps_ - 1, 1), q_width() + k_width() + v_width()}, DType::F32}};
     }
     long long q_width() const { return static_cast<long long>(shape_.heads) * shape_.head_dim; }
     long long k_width() const { return static_cast<long long>(shape_.kv_heads) * shape_.head_dim; }
@@ -1559,9 +1690,16 @@ public:
             specs.push_back({"r2", vec(shape_.heads, "around_one")});
         }
         if (gated_) specs.push_back({"g", matrix(o_width(), width_)});
+        if (taps_ > 0) {
+            auto taps = [&](long long n) { return WeightSpec{{n, taps_}, "vector", "normal", {}}; };
+            specs.push_back({"q_conv", taps(q_width())});
+            specs.push_back({"k_conv", taps(k_width())});
+            specs.push_back({"v_conv", taps(v_width())});
+        }
         return specs;
     }
     void load(const PartTensors& t, Runtime&) override {
+        if (taps_ > 0) conv_w_ = concat_rows({get(t, "q_conv"), get(t, "k_conv"), get(t, "v_conv")});
         std::vector<std::pair<std::shared_ptr<DeviceTensor>, bool>> pieces{{get(t, "q"), false}, {get(t, "k"), false}, {get(t, "v"), false}};
         if (gated_) pieces.push_back({get(t, "g"), false});
         const Stacked in = stack_projections(pieces, "biased_attention");
@@ -1580,10 +1718,22 @@ public:
         Tensor proj = rt.ws.buf("battn_proj", rt.dtype, {T, w_in_->view.shape[0]});
         rt.ops.linear(x, w_in_->view, proj, nullptr, rt.ws);
         // every row's keys and values are in their pages before any row attends
-        rt.ops.kv_store(proj.cols(col_k_, k_width()), proj.cols(col_v_, v_width()), batch, *cache.kv);
+        Tensor q = proj.cols(0, q_width());
+        if (taps_ > 0 || position_) {
+            // convolutions continuing from the request's saved rows, rotation, queries to a buffer of their own
+            PositionEncoding::Tables tables;
+            if (position_) tables = position_->tables(rt);
+            const Tensor* inv_freq = tables.inv_freq.defined() ? &tables.inv_freq : nullptr;
+            q = rt.ws.buf("battn_q", rt.dtype, {T, q_width()});
+            const Tensor* state = taps_ > 0 ? &cache.states.at("conv") : nullptr;
+            rt.ops.conv_rope_store(proj, taps_ > 0 ? &conv_w_->view : nullptr, state, taps_, inv_freq, tables.rotary_dim, tables.pairing,
+                                   q, shape_.heads, batch, *cache.kv);
+        } else {
+            rt.ops.kv_store(proj.cols(col_k_, k_width()), proj.cols(col_v_, v_width()), batch, *cache.kv);
+        }
         Tensor attended = rt.ws.buf("battn_out", rt.dtype, {T, o_width()});
         Tensor gate = gated_ ? proj.cols(col_g_, o_width()) : Tensor();
-        rt.ops.biased_attention(proj.cols(0, q_width()), attended, shape_, r1_ ? &r1_->view : nullptr, r2_ ? &r2_->view : nullptr,
+        rt.ops.biased_attention(q, attended, shape_, r1_ ? &r1_->view : nullptr, r2_ ? &r2_->view : nullptr,
                                 gated_ ? &gate : nullptr, batch, *cache.kv, rt.ws);
         Tensor out = rt.ws.buf("battn_mixer_out", rt.dtype, {T, width_});
         rt.ops.linear(attended, w_o_->view, out, nullptr, rt.ws);
@@ -1594,7 +1744,9 @@ private:
     long long width_ = 0, col_k_ = 0, col_v_ = 0, col_g_ = 0;
     Ops::ScoreShape shape_;
     bool distance_bias_ = false, gated_ = false;
-    std::shared_ptr<DeviceTensor> w_in_, w_o_, r1_, r2_;
+    int taps_ = 0;
+    std::unique_ptr<PositionEncoding> position_;
+    std::shared_ptr<DeviceTensor> w_in_, w_o_, r1_, r2_, conv_w_;
 };
 
 // ---------------------------------------------------------------------------- real-gated linear recurrent unit
@@ -1996,6 +2148,7 @@ void register_builtin_parts() {
     r.parts["norm"]["rmsnorm"] = factory_of<RmsNorm>();
     r.parts["norm"]["identity"] = factory_of<IdentityNorm>();
     r.parts["norm"]["layernorm"] = factory_of<LayerNorm>();
+    r.parts["norm"]["dynamic_tanh"] = factory_of<DynamicTanh>();
     r.parts["position"]["rope"] = factory_of<Rope>();
     r.parts["position"]["none"] = factory_of<NoPosition>();
     r.parts["mixer"]["gqa_attention"] = factory_of<GqaAttention>();
@@ -2004,6 +2157,7 @@ void register_builtin_parts() {
     r.parts["mixer"]["sigmoid_attention"] = factory_of<SigmoidAttention>();
     r.parts["mixer"]["gated_delta_rule"] = factory_of<GatedDeltaRule>();
     r.parts["reinjection"]["linear_concat"] = factory_of<LinearReinjection>();
+    r.parts["reinjection"]["add_rows"] = factory_of<AdditiveReinjection>();
     r.parts["mixer"]["biased_attention"] = factory_of<BiasedAttention>();
     r.parts["mixer"]["linear_recurrent_unit"] = factory_of<LinearRecurrentUnit>();
     r.parts["mixer"]["normed_pair"] = factory_of<NormedPair>();

@@ -71,8 +71,9 @@ public:
 class Reinjection : public Part {
 public:
     using Part::Part;
-    // h [T, width] 32-bit, the stream, is replaced; x0 [T, width] 32-bit are the embedding's rows
-    virtual void forward(const Tensor& h, const Tensor& x0, Runtime& rt) = 0;
+    // h [T, width] 32-bit, the stream, is replaced; x0 [T, width] 32-bit are the embedding's rows;
+    // pass: which run of the looped range begins (RunStep::pass)
+    virtual void forward(const Tensor& h, const Tensor& x0, Runtime& rt, int pass) = 0;
 };
 
 // What the rows' token ids add to the residual stream after a layer's sub-layers.

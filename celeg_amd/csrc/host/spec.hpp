@@ -18,10 +18,11 @@
 //           "ffn_post_norm"; a layer may name a "token_input" (a part that adds something made from the
 //           rows' token ids to the stream after the sub-layers) and a "depth_mix" (a part that replaces
 //           the stream behind the layer by a mixture of the results of all entries of the run order so
-//           far, the embedding's rows first)
+//           far, the embedding's rows first); "residual_scale" (1 if absent) multiplies what a sub-layer adds to
+//           the stream, in arrangements that know it ("sandwich_norm")
 //   model: {"architecture", "vocab_size", "hidden_size", "max_context", "streams" (residual
 //           streams per row, 1 if absent), "embedding": part,
-//           "layers": [layer], "order": [{"layer": i, "kv_from": j or null, "reinject": bool}],
+//           "layers": [layer], "order": [{"layer": i, "kv_from": j or null, "reinject": bool, "pass": n}],
 //           "reinjection": part (how the embedding's rows come back into the stream before the
 //           entries of the order that say "reinject"; absent: never),
 //           "final_norm": part, "head": part, "eos_token_ids": [..], "bos_token_id"}
@@ -92,6 +93,8 @@ struct LayerSpec {
     // layer is mixed from the results of the entries run so far (kind empty: none)
     PartSpec token_input, depth_mix;
     std::string arrangement = "pre_norm";
+    // what a sub-layer's (normed) output is multiplied by as it is added to the stream
+    double residual_scale = 1.0;
 };
 
 // One entry of the run order.  `layer` indexes ModelSpec::layers (a layer may be named more
@@ -104,6 +107,9 @@ struct RunStep {
     // before this entry runs, the stream is replaced by the model's reinjection part's mixture of
     // the stream and the embedding's rows
     bool reinject = false;
+    // which run of a looped range of layers this entry belongs to (0 where nothing is looped): what a
+    // reinjection that differs from run to run is told
+    int pass = 0;
 };
 
 struct ModelSpec {
@@ -148,12 +154,14 @@ struct ModelSpec {
             if (!l.ffn_post_norm.kind.empty()) lj.set("ffn_post_norm", l.ffn_post_norm.to_json());
             if (!l.token_input.kind.empty()) lj.set("token_input", l.token_input.to_json());
             if (!l.depth_mix.kind.empty()) lj.set("depth_mix", l.depth_mix.to_json());
+            if (l.residual_scale != 1.0) lj.set("residual_scale", l.residual_scale);
             ls.push(lj);
         }
         Json ord = Json::array();
         for (const auto& s : order) {
             Json e = Json::object().set("layer", s.layer).set("kv_from", s.kv_from ? Json(*s.kv_from) : Json());
             if (s.reinject) e.set("reinject", true);
+            if (s.pass) e.set("pass", s.pass);
             ord.push(e);
         }
         Json out = Json::object();
@@ -192,6 +200,7 @@ struct ModelSpec {
             if (!l["token_input"].is_null()) ls.token_input = PartSpec::from_json(l["token_input"], where + ".token_input");
             if (!l["depth_mix"].is_null()) ls.depth_mix = PartSpec::from_json(l["depth_mix"], where + ".depth_mix");
             ls.arrangement = l.get_string("arrangement", "pre_norm");
+            ls.residual_scale = l.get_double("residual_scale", 1.0);
             m.layers.push_back(std::move(ls));
         }
         if (j["order"].is_array()) {
@@ -200,6 +209,7 @@ struct ModelSpec {
                 step.layer = static_cast<int>(s.is_object() ? s.get_int("layer", -1) : s.as_int());
                 if (s.is_object() && !s["kv_from"].is_null()) step.kv_from = static_cast<int>(s["kv_from"].as_int());
                 if (s.is_object()) step.reinject = s.get_bool("reinject", false);
+                if (s.is_object()) step.pass = static_cast<int>(s.get_int("pass", 0));
                 m.order.push_back(step);
             }
         } else {

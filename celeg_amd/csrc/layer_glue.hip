@@ -1,6 +1,7 @@
 // What holds a layer together besides its norms: activations with a bias, sums into the 32-bit
 // residual stream, a per-layer token input, the mean of several normed branches, and the
-// weighted sum over the results of all earlier layers.  All arithmetic is 32-bit; T is the
+// weighted sum over the results of all earlier layers, what a stream takes in before a run of a looped
+// range, and logits bent by a tanh.  All arithmetic is 32-bit; T is the
 // run's dtype of the branch rows.
 #include "common.h"
 
@@ -91,6 +92,24 @@ __global__ void depth_mix_kernel(float* __restrict__ history, size_t entry_strid
     h[at] = fmaf(w[n - 1], last, sum);
 }
 
+// h[t, :] += (rows[t, :] +) vec, all 32-bit: what a stream takes in before a run of a looped range
+__global__ void stream_add_kernel(float* __restrict__ h, const float* __restrict__ rows, const float* __restrict__ vec, int width) {
+    const int t = blockIdx.y;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= width) return;
+    const size_t at = static_cast<size_t>(t) * width + c;
+    float v = h[at];
+    if (rows) v += rows[at];
+    if (vec) v += vec[c];
+    h[at] = v;
+}
+
+// x <- cap * tanh(x / cap), 32-bit
+__global__ void softcap_kernel(float* __restrict__ x, size_t n, float cap) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
 }  // namespace
 
 #define LG_BY_DTYPE(kernel, grid, block, ...)                                                      \
@@ -142,5 +161,19 @@ extern "C" int celeg_depth_mix(float* history, size_t entry_stride, float* h, co
     if (rows <= 0 || n <= 0) return 0;
     dim3 grid((width + 255) / 256, rows), block(256);
     hipLaunchKernelGGL(depth_mix_kernel, grid, block, 0, stream, history, entry_stride, h, w, n, width);
+    return CELEG_LAUNCH_RESULT();
+}
+
+extern "C" int celeg_stream_add(float* h, const float* rows, const float* vec, int n_rows, int width, hipStream_t stream) {
+    if (n_rows <= 0 || (!rows && !vec)) return 0;
+    dim3 grid((width + 255) / 256, n_rows), block(256);
+    hipLaunchKernelGGL(stream_add_kernel, grid, block, 0, stream, h, rows, vec, width);
+    return CELEG_LAUNCH_RESULT();
+}
+
+extern "C" int celeg_softcap(float* x, size_t n, float cap, hipStream_t stream) {
+    if (n == 0) return 0;
+    if (!(cap > 0.f)) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(softcap_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, stream, x, n, cap);
     return CELEG_LAUNCH_RESULT();
 }

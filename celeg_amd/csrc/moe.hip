@@ -12,10 +12,23 @@
 #define MOE_MAX_PER_LANE 8        // experts <= 512
 
 // ---------------------------------------------------------------- route
-// One wavefront per row.  score 0: sigmoid of the logit; 1: softmax over all experts.
-// The chosen experts' scores are the weights; with `renorm` they are divided by their sum.
-__device__ __forceinline__ void route_row(const float* z, int experts, int top, int score, int renorm, int* ids,
-                                          float* weights) {
+// How a row's experts are chosen and weighted.  score 0: sigmoid of the logit; 1: softmax over all
+// experts.  groups > 1: the experts form `groups` equal runs of neighbours, a run's score is the sum of
+// its two largest scores, and only experts of the `keep` best runs (the lower run among equal ones) can be
+// chosen.  The chosen experts' scores are the weights; with `renorm` they are divided by their sum plus
+// renorm_eps; then times `scale`.
+struct MoeRule {
+    int experts, top, score, renorm, groups, keep;
+    float renorm_eps, scale;
+};
+
+__device__ __forceinline__ float route_score(float z, int score, float zmax, float denom) {
+    return score == 1 ? expf(z - zmax) / denom : 1.0f / (1.0f + expf(-z));
+}
+
+// One wavefront per row.
+__device__ __forceinline__ void route_row(const float* z, const MoeRule& rule, int* ids, float* weights) {
+    const int experts = rule.experts, top = rule.top, score = rule.score;
     const int lane = threadIdx.x & 63;
     float v[MOE_MAX_PER_LANE];
     float zmax = -INFINITY;
@@ -33,6 +46,52 @@ __device__ __forceinline__ void route_row(const float* z, int experts, int top, 
         for (int j = 0; j < MOE_MAX_PER_LANE; ++j)
             if (lane + j * CELEG_WAVE < experts) s += expf(v[j] - zmax);
         denom = wave_sum(s);
+    }
+    if (rule.groups > 1) {
+        // every run's two largest scores (the largest logits give them), their sum in lane g of `mine`
+        const int per = experts / rule.groups;
+        float mine = -INFINITY;
+        for (int g = 0; g < rule.groups; ++g) {
+            float first = -INFINITY, second = -INFINITY;      // this lane's two largest logits of run g
+#pragma unroll
+            for (int j = 0; j < MOE_MAX_PER_LANE; ++j) {
+                const int e = lane + j * CELEG_WAVE;
+                if (e < experts && e / per == g) {
+                    if (v[j] > first) { second = first; first = v[j]; }
+                    else if (v[j] > second) second = v[j];
+                }
+            }
+#pragma unroll
+            for (int off = CELEG_WAVE / 2; off > 0; off >>= 1) {
+                const float of = __shfl_xor(first, off, CELEG_WAVE), os = __shfl_xor(second, off, CELEG_WAVE);
+                const float hi = fmaxf(first, of), lo = fminf(first, of);
+                second = fmaxf(lo, fmaxf(second, os));
+                first = hi;
+            }
+            float sum = route_score(first, score, zmax, denom);
+            if (per > 1) sum += route_score(second, score, zmax, denom);
+            if (lane == g) mine = sum;
+        }
+        // the `keep` best runs stay; the experts of the others leave the choice
+        unsigned long long kept = 0ull;
+        for (int k = 0; k < rule.keep; ++k) {
+            float best = mine;
+            int best_g = lane < rule.groups ? lane : 0x7fffffff;
+            if (lane >= rule.groups) best = -INFINITY;
+#pragma unroll
+            for (int off = CELEG_WAVE / 2; off > 0; off >>= 1) {
+                const float ob = __shfl_xor(best, off, CELEG_WAVE);
+                const int og = __shfl_xor(best_g, off, CELEG_WAVE);
+                if (ob > best || (ob == best && og < best_g)) { best = ob; best_g = og; }
+            }
+            kept |= 1ull << best_g;
+            if (lane == best_g) mine = -INFINITY;
+        }
+#pragma unroll
+        for (int j = 0; j < MOE_MAX_PER_LANE; ++j) {
+            const int e = lane + j * CELEG_WAVE;
+            if (e < experts && !((kept >> (e / per)) & 1ull)) v[j] = -INFINITY;
+        }
     }
     float total = 0.f;
     for (int k = 0; k < top; ++k) {
@@ -53,21 +112,20 @@ __device__ __forceinline__ void route_row(const float* z, int experts, int top, 
 #pragma unroll
         for (int j = 0; j < MOE_MAX_PER_LANE; ++j)
             if (lane + j * CELEG_WAVE == best_e) v[j] = -INFINITY;
-        const float s = score == 1 ? expf(best - zmax) / denom : 1.0f / (1.0f + expf(-best));
+        const float s = route_score(best, score, zmax, denom);
         total += s;
         if (lane == 0) {
             ids[k] = best_e;
             weights[k] = s;
         }
     }
-    if (renorm && lane == 0)
-        for (int k = 0; k < top; ++k) weights[k] /= total;
+    if (lane == 0 && (rule.renorm || rule.scale != 1.0f))
+        for (int k = 0; k < top; ++k) weights[k] = (rule.renorm ? weights[k] / (total + rule.renorm_eps) : weights[k]) * rule.scale;
 }
 
-__global__ void moe_route_kernel(const float* __restrict__ logits, int experts, int top, int score, int renorm,
-                                 int* __restrict__ ids, float* __restrict__ weights) {
+__global__ void moe_route_kernel(const float* __restrict__ logits, MoeRule rule, int* __restrict__ ids, float* __restrict__ weights) {
     const size_t t = blockIdx.x;
-    route_row(logits + t * experts, experts, top, score, renorm, ids + t * top, weights + t * top);
+    route_row(logits + t * rule.experts, rule, ids + t * rule.top, weights + t * rule.top);
 }
 
 // The router's product and the choice in one kernel: a workgroup takes four rows, keeps them in LDS
@@ -76,8 +134,8 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int experts, 
 #define ROUTE_ROWS 4
 template <typename TX>
 __global__ __launch_bounds__(256) void moe_router_kernel(const TX* __restrict__ x, const float* __restrict__ w, int rows,
-                                                         int width, int experts, int top, int score, int renorm,
-                                                         int* __restrict__ ids, float* __restrict__ weights) {
+                                                         int width, MoeRule rule, int* __restrict__ ids, float* __restrict__ weights) {
+    const int experts = rule.experts, top = rule.top;
     extern __shared__ float router_lds[];        // ROUTE_ROWS rows of width, then ROUTE_ROWS rows of logits
     float* xs = router_lds;
     float* zs = router_lds + ROUTE_ROWS * width;
@@ -119,8 +177,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(const TX* __restrict__ 
     __syncthreads();
     const int t = row0 + wave;
     if (t < rows)
-        route_row(zs + wave * experts, experts, top, score, renorm, ids + static_cast<size_t>(t) * top,
-                  weights + static_cast<size_t>(t) * top);
+        route_row(zs + wave * experts, rule, ids + static_cast<size_t>(t) * top, weights + static_cast<size_t>(t) * top);
 }
 
 // ---------------------------------------------------------------- plan
@@ -288,10 +345,11 @@ __global__ __launch_bounds__(256, 2) void moe_product_mfma_kernel(const __bf16* 
 }
 
 // ---------------------------------------------------------------- combine
-// out[t, :] = sum_k (weight of entry (t, k)) * y[place_of[t * top + k], :], summed in 32-bit
+// out[t, :] = (base[t, :] +) sum_k (weight of entry (t, k)) * y[place_of[t * top + k], :], summed in 32-bit
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ place_of,
-                                   const float* __restrict__ weights, T* __restrict__ out, int top, int width) {
+                                   const float* __restrict__ weights, const T* __restrict__ base, T* __restrict__ out, int top,
+                                   int width) {
     const int t = blockIdx.x;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         float acc = 0.f;
@@ -300,36 +358,45 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
             const float v = to_float(y[static_cast<size_t>(place_of[entry]) * width + i]);
             acc += weights ? weights[entry] * v : v;
         }
+        if (base) acc += to_float(base[static_cast<size_t>(t) * width + i]);
         out[static_cast<size_t>(t) * width + i] = from_float<T>(acc);
     }
 }
 
 // ---------------------------------------------------------------- entry points
-extern "C" int celeg_moe_route(const float* logits, int rows, int experts, int top, int score, int renorm, int* ids,
-                               float* weights, hipStream_t stream) {
+// whether a rule is one the routing kernels take: groups that divide the experts evenly, at most 64 of them,
+// and enough experts in the kept ones
+static bool moe_rule_ok(const MoeRule& r) {
+    if (r.experts <= 0 || r.experts > MOE_MAX_PER_LANE * CELEG_WAVE || r.top <= 0 || r.top > r.experts) return false;
+    if (r.groups < 1 || r.groups > CELEG_WAVE || r.experts % r.groups || r.keep < 1 || r.keep > r.groups) return false;
+    return r.top <= r.keep * (r.experts / r.groups);
+}
+
+extern "C" int celeg_moe_route(const float* logits, int rows, int experts, int top, int score, int renorm, int groups, int keep,
+                               float renorm_eps, float scale, int* ids, float* weights, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (experts <= 0 || experts > MOE_MAX_PER_LANE * CELEG_WAVE || top <= 0 || top > experts)
-        return static_cast<int>(hipErrorInvalidValue);
-    hipLaunchKernelGGL(moe_route_kernel, dim3(rows), dim3(CELEG_WAVE), 0, stream, logits, experts, top, score, renorm, ids,
-                       weights);
+    const MoeRule rule{experts, top, score, renorm, groups, keep, renorm_eps, scale};
+    if (!moe_rule_ok(rule)) return static_cast<int>(hipErrorInvalidValue);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(rows), dim3(CELEG_WAVE), 0, stream, logits, rule, ids, weights);
     return CELEG_LAUNCH_RESULT();
 }
 
 // rows of a tile: 64 where every product of the plan runs on the matrix cores, else 32
 // x [rows, width] (32-bit or bfloat16) times the router's 32-bit matrix w [experts, width], then the choice
 extern "C" int celeg_moe_router(const void* x, int x_dtype, const float* w, int rows, int width, int experts, int top,
-                                int score, int renorm, int* ids, float* weights, hipStream_t stream) {
+                                int score, int renorm, int groups, int keep, float renorm_eps, float scale, int* ids,
+                                float* weights, hipStream_t stream) {
     if (rows <= 0) return 0;
     const size_t lds = static_cast<size_t>(ROUTE_ROWS) * (width + experts) * sizeof(float);
-    if (experts <= 0 || experts > MOE_MAX_PER_LANE * CELEG_WAVE || top <= 0 || top > experts || lds > 64 * 1024)
-        return static_cast<int>(hipErrorInvalidValue);
+    const MoeRule rule{experts, top, score, renorm, groups, keep, renorm_eps, scale};
+    if (!moe_rule_ok(rule) || lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
     dim3 grid((rows + ROUTE_ROWS - 1) / ROUTE_ROWS);
     if (x_dtype == CELEG_F32)
         hipLaunchKernelGGL(moe_router_kernel<float>, grid, dim3(256), lds, stream, static_cast<const float*>(x), w, rows, width,
-                           experts, top, score, renorm, ids, weights);
+                           rule, ids, weights);
     else
         hipLaunchKernelGGL(moe_router_kernel<bf16>, grid, dim3(256), lds, stream, static_cast<const bf16*>(x), w, rows, width,
-                           experts, top, score, renorm, ids, weights);
+                           rule, ids, weights);
     return CELEG_LAUNCH_RESULT();
 }
 
@@ -387,14 +454,15 @@ extern "C" int celeg_moe_product(const void* a, const void* w, void* out, int dt
     return CELEG_LAUNCH_RESULT();
 }
 
-extern "C" int celeg_moe_combine(const void* y, int dtype, const int* place_of, const float* weights, void* out, int rows,
-                                 int top, int width, hipStream_t stream) {
+// base: rows [rows, width] added to the sum (what every row gets besides its experts), or null
+extern "C" int celeg_moe_combine(const void* y, int dtype, const int* place_of, const float* weights, const void* base, void* out,
+                                 int rows, int top, int width, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (dtype == CELEG_F32)
         hipLaunchKernelGGL(moe_combine_kernel<float>, dim3(rows), dim3(256), 0, stream, static_cast<const float*>(y),
-                           place_of, weights, static_cast<float*>(out), top, width);
+                           place_of, weights, static_cast<const float*>(base), static_cast<float*>(out), top, width);
     else
         hipLaunchKernelGGL(moe_combine_kernel<bf16>, dim3(rows), dim3(256), 0, stream, static_cast<const bf16*>(y), place_of,
-                           weights, static_cast<bf16*>(out), top, width);
+                           weights, static_cast<const bf16*>(base), static_cast<bf16*>(out), top, width);
     return CELEG_LAUNCH_RESULT();
 }

@@ -8,12 +8,20 @@
 //
 // Layer norm: (x - mean) / sqrt(var + eps) * w + b with var the mean of the squared deviations
 // from the mean (two passes over the row, which is staged in LDS).  RMS norm:
-// x / sqrt(mean(x^2) + eps) * w.  The bias is optional in both.
+// x / sqrt(mean(x^2) + eps) * w.  The bias is optional in both.  "Dynamic tanh": tanh(alpha * x) * w + b
+// with one number alpha, no statistic of the row at all.  A norm's `gain` multiplies what it gives
+// as a whole (a block that adds m * post(y)).
 #include "common.h"
 
 #include "norm_params.h"
 
 namespace {
+
+// one value through a norm whose statistics are (shift, factor)
+__device__ __forceinline__ float normed_value(float x, const CelegNorm& n, float shift, float factor, float w, float b) {
+    const float v = n.mode == CELEG_NORM_TANH ? tanhf(n.alpha * x) : (x - shift) * factor;
+    return (v * w + b) * n.gain;
+}
 
 // the statistics of `row` (LDS, width floats) for a norm of this mode: (shift, factor) such that
 // the normalised value is (x - shift) * factor
@@ -50,9 +58,7 @@ __global__ __launch_bounds__(256) void norm_step_kernel(float* __restrict__ h, c
         float shift, factor;
         row_stats(row, width, post.mode, post.eps, scratch, shift, factor);
         for (int i = threadIdx.x; i < width; i += blockDim.x) {
-            float v = (row[i] - shift) * factor;
-            if (post.w) v *= post.w[i];
-            if (post.b) v += post.b[i];
+            float v = normed_value(row[i], post, shift, factor, post.w ? post.w[i] : 1.f, post.b ? post.b[i] : 0.f);
             v += h[src + i];
             row[i] = v;                 // (its own element: no other thread reads it before the barrier)
             if (write_back) h[src + i] = v;
@@ -66,10 +72,7 @@ __global__ __launch_bounds__(256) void norm_step_kernel(float* __restrict__ h, c
     row_stats(row, width, pre.mode, pre.eps, scratch, shift, factor);
     TO* dst = out + static_cast<size_t>(r) * width;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        float v = (row[i] - shift) * factor;
-        if (pre.w) v *= pre.w[i];
-        if (pre.b) v += pre.b[i];
-        dst[i] = from_float<TO>(v);
+        dst[i] = from_float<TO>(normed_value(row[i], pre, shift, factor, pre.w ? pre.w[i] : 1.f, pre.b ? pre.b[i] : 0.f));
     }
 }
 
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(256) void norm_step_reg_kernel(float* __restrict__ 
         reg_stats<NV>(yv, in, width, post.mode, post.eps, scratch, shift, factor);
 #pragma unroll
         for (int k = 0; k < NV; ++k) {
-            hv[k] = ((yv[k] - shift) * factor * pw[k] + pb[k]) + hv[k];
+            hv[k] = normed_value(yv[k], post, shift, factor, pw[k], pb[k]) + hv[k];
             if (write_back && in[k]) h[src + threadIdx.x + 256 * k] = hv[k];
         }
     }
@@ -134,7 +137,7 @@ __global__ __launch_bounds__(256) void norm_step_reg_kernel(float* __restrict__ 
     TO* dst = out + static_cast<size_t>(r) * width;
 #pragma unroll
     for (int k = 0; k < NV; ++k)
-        if (in[k]) dst[threadIdx.x + 256 * k] = from_float<TO>((hv[k] - shift) * factor * nw[k] + nb[k]);
+        if (in[k]) dst[threadIdx.x + 256 * k] = from_float<TO>(normed_value(hv[k], pre, shift, factor, nw[k], nb[k]));
 }
 
 template <typename TO>
