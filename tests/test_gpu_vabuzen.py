@@ -1,0 +1,779 @@
+"""The Vabuzen design in the engine against the plain implementation (``plain_vabuzen.py``):
+each mechanism alone through the step function (the attention behind short convolutions with its
+window, kept first keys and the one in the softmax's denominator; the attention over compressed rows;
+routed experts chosen inside the best groups with a shared expert; the dense feed-forward; the block of
+dynamic tanh norms with its factor), whole models of several shapes in every way of cutting and
+batching, inputs made so that a far key, a kept first key, a window that is one key off or a lost
+convolution state shows, long decoding while the window passes over decoded tokens, pages and slots
+used again, and greedy generation through the engine's entry point and scheduler.  Sizes differ from
+model to model in every number and include values that make mechanisms degenerate: one query head per
+key head and all on one, no convolution and one tap, rotation of a part of a head and of none, windows
+of one key and none, nothing kept and more kept than a page holds, one group of experts and as many
+groups as kept, one expert a token, no shared expert, a layer without feed-forward, a loop of one run,
+over the first layers, over all and none, factors of one and others, no bend of the logits, widths that
+are no multiple of 16.
+"""
+import json
+import os
+
+import pytest
+import torch
+
+import plain_vabuzen as plain
+from helpers import (EngineDriver, assert_close_f32, mixed_schedule, peak_tokens, portions_schedule, random_tokens,
+                     tail_decode_schedule, whole_schedule)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+STD = 0.08
+
+
+def assert_close(got, ref, dtype, what=""):
+    """32-bit: the shared bound (1e-4 of the largest logit).  bfloat16: relative RMS error <= 4e-2, and
+    every row's max |d| <= 8e-2 * max |ref| but for one row in fifty (at least one): a router that hangs
+    on a close call between two experts, or between two groups, changes its choice with the rounding of
+    its input; such rows are the same in every schedule.  The faults these tests look for move many rows
+    by tens of percent, and the 32-bit runs of the same schedules hold every row to 1e-4."""
+    if dtype in ("float32", torch.float32):
+        return assert_close_f32(got, ref, what)
+    got, ref = torch.as_tensor(got).double(), torch.as_tensor(ref).double()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite logits"
+    d = got - ref
+    rel = float(d.pow(2).mean().sqrt() / ref.pow(2).mean().sqrt())
+    rows = d.abs().reshape(-1, d.shape[-1]).max(-1).values / ref.abs().max()
+    over = int((rows > 8e-2).sum())
+    assert rel <= 4e-2 and over <= max(1, rows.numel() // 50), \
+        f"{what}: rel rms {rel:.3e} (<= 4e-2), {over} of {rows.numel()} rows over 8e-2 of the largest logit, worst {float(rows.max()):.3e}"
+
+
+def dense(ff):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts, top, ff, groups=None, scale=None, shared=None):
+    router = {"experts": experts, "top": top}
+    if groups:
+        router["groups"] = {"count": groups[0], "keep": groups[1]}
+    if scale is not None:
+        router["scale"] = scale
+    out = {"kind": "moe", "expert": {"ff": ff}, "router": router}
+    if shared:
+        out["shared"] = {"ff": shared}
+    return out
+
+
+def attention(heads, kv_heads, dim, vdim, scale, conv, rot, mask, mlp):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if conv:
+        m["conv"] = conv
+    if rot:
+        m["rot"] = {"base": rot[0], "dims": rot[1]}
+    if mask:
+        m["mask"] = {"size": mask[0], "keep_first": mask[1]}
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def latent(heads, dim, rot_dim, vdim, rank, scale, base, mlp):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": rank, "scale": scale}
+    if rot_dim:
+        m["rot"] = {"base": base, "dims": rot_dim}
+    return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+
+# heads the matrix cores take (keys and values of different sizes), a loop of two runs in the middle
+V1 = {"architecture": "Vabuzen", "vocab": 310, "width": 96, "norm": {"eps": 1e-5}, "residual_mult": 0.7, "logit_softcap": 8.0,
+      "loop": {"start": 1, "stop": 3, "times": 2},
+      "layers": [latent(4, 16, 16, 32, 48, 0.18, 20000.0, moe(8, 2, 32, (4, 2), 1.5, 48)),
+                 attention(4, 2, 32, 64, 0.2, 3, (1000.0, 16), (24, 3), dense(80)),
+                 latent(3, 24, 8, 16, 32, 0.2, 500.0, None),
+                 attention(3, 3, 64, 32, 0.12, 4, (10000.0, 64), (33, 20), moe(6, 3, 24, (2, 1), 2.5, None))]}
+# a width that is no multiple of 16, heads no matrix-core kernel takes, all query heads on one key head, no
+# convolution, one tap, no rotation, no window, a window of one key, a loop of one run over the first layers,
+# no bend of the logits, a factor of one (absent), one expert a token, every expert in one group
+V2 = {"architecture": "Vabuzen", "vocab": 211, "width": 72, "norm": {"eps": 3e-6}, "loop": {"start": 0, "stop": 2, "times": 1},
+      "layers": [attention(5, 1, 12, 20, 0.3, 0, None, None, moe(5, 1, 24, None, None, 40)),
+                 latent(2, 12, 0, 20, 24, 0.3, 0.0, dense(40)),
+                 attention(2, 2, 8, 8, 0.35, 1, (50.0, 8), (1, 0), None),
+                 attention(6, 3, 10, 14, 0.3, 5, (300.0, 4), (7, 9), moe(4, 4, 16, (1, 1), 0.5, 24))]}
+# heads of 128 and 96, the loop over every layer three times, more kept first keys than a page holds, as many
+# kept groups as groups
+V3 = {"architecture": "Vabuzen", "vocab": 260, "width": 128, "norm": {"eps": 1e-4}, "residual_mult": 1.3, "logit_softcap": 30.0,
+      "loop": {"start": 0, "stop": 3, "times": 3},
+      "layers": [attention(2, 1, 128, 96, 0.09, 2, (500000.0, 32), (50, 18), moe(9, 2, 48, (3, 3), 1.0, 64)),
+                 latent(8, 32, 32, 32, 64, 0.125, 10000.0, dense(64)),
+                 attention(4, 2, 96, 128, 0.1, 4, (10000.0, 96), (16, 1), dense(96))]}
+MODELS = {"V1": (V1, 41), "V2": (V2, 42), "V3": (V3, 43)}
+LENGTHS = {"V1": [40, 57, 90, 128, 65, 33], "V2": [45, 130, 64, 100, 17, 33], "V3": [31, 32, 150, 64, 49, 80]}
+SCHEDULES = {"whole": whole_schedule, "tail12": lambda reqs: tail_decode_schedule(reqs, tail=12),
+             "portions": portions_schedule, "mixed": mixed_schedule}
+
+
+def write_model(folder, cfg, seed, storage=torch.float32, std=STD, replace=None, change=None):
+    """A model folder of random tensors for ``cfg``; ``replace``: name -> tensor, ``change``:
+    name -> function of the drawn tensor."""
+    from celeg_amd import native
+    from celeg_amd.weights import random_tensors
+    from celeg_amd.weights.safetensors_io import write_safetensors
+    expected = native.describe_config(cfg)["expected_tensors"]
+    tensors = random_tensors(expected, seed, std, torch.float32)
+    for name in tensors:
+        # the norms' biases, the vectors of the runs and the convolutions' taps large enough to matter
+        if name.endswith(".b") or name == "loop.step":
+            tensors[name] = tensors[name] * 3.0
+        if name.endswith(".conv"):
+            tensors[name] = tensors[name] * 6.0
+    for name, t in (replace or {}).items():
+        assert tensors[name].shape == t.shape, name
+        tensors[name] = t.float()
+    for name, fn in (change or {}).items():
+        tensors[name] = fn(tensors[name])
+    tensors = {k: v.to(storage).contiguous() for k, v in tensors.items()}
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as fh:
+        json.dump(cfg, fh)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    return str(folder)
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    made = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in made:
+            cfg, seed = MODELS[name]
+            storage = torch.float32 if dtype == "float32" else torch.bfloat16
+            made[(name, dtype)] = write_model(tmp_path_factory.mktemp(f"{name}_{dtype}"), cfg, seed, storage)
+        return made[(name, dtype)]
+    return get
+
+
+_plain = {}
+
+
+def requests_of(name):
+    cfg, seed = MODELS[name]
+    return {f"r{i}": random_tokens(cfg["vocab"], n, seed=100 * seed + i) for i, n in enumerate(LENGTHS[name])}
+
+
+def plain_logits(folder, key, requests):
+    if key not in _plain:
+        cfg, W = plain.load_model_folder(folder)
+        _plain[key] = {rid: plain.model_logits(cfg, W, toks) for rid, toks in requests.items()}
+    return _plain[key]
+
+
+def load(folder, dtype, steps, max_requests=4, **kw):
+    from celeg_amd.engine import load_model
+    max_tokens = peak_tokens(steps)
+    lm = load_model(folder, dtype=dtype, device=DEV, page_tokens=16, n_pages=max_tokens // 16, max_requests=max_requests,
+                    max_context=max_tokens, max_batched_tokens=max(max_tokens, 64), **kw)
+    return lm, max_tokens
+
+
+@pytest.mark.parametrize("mode", list(SCHEDULES))
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(MODELS))
+def test_engine_matches_plain(folders, name, dtype, mode):
+    """Whole prompts; prefill then 12 tokens one by one; portions down to two tokens (and single
+    ones) that cross page borders; four live requests with pages and slots used again."""
+    folder = folders(name, dtype)
+    reqs = requests_of(name)
+    steps = SCHEDULES[mode](reqs)
+    lm, max_tokens = load(folder, dtype, steps)
+    got = EngineDriver(lm).run(steps)
+    ref = plain_logits(folder, (name, dtype), reqs)
+    for rid in reqs:
+        assert_close(got[rid], ref[rid], dtype, f"{name}/{dtype}/{mode}/{rid}")
+    lm.cache.check()
+    assert lm.cache.n_free_slots == 4 and lm.cache.free_pages() == [max_tokens // 16] * len(lm.cache.free_pages())
+    paths = lm.paths()
+    assert paths["attention_biased"] > 0 and paths["attention_latent"] > 0 and paths["routed_experts"] > 0
+    if dtype == "bfloat16" and name != "V2":
+        assert paths["attention_biased_rows"] + paths["attention_biased_decode"] > 0     # the matrix cores took these heads
+
+
+@pytest.mark.parametrize("name", ["V1", "V2", "V3"])
+def test_residual_stream_after_every_run_of_a_layer(folders, tmp_path, monkeypatch, name):
+    """32-bit: the stream behind each entry of the run order as CELEG_DUMP_HIDDEN writes it, for a
+    prompt's portion and two single tokens, against the plain layers: the first that differs is where a
+    fault lies (what is added before a run of the looped range shows in that run's first entry)."""
+    import numpy as np
+    from celeg_amd.engine import StepEntry, load_model
+    cfg, _ = MODELS[name]
+    folder = folders(name, "float32")
+    _, W = plain.load_model_folder(folder)
+    toks = random_tokens(cfg["vocab"], 23, seed=2)
+    after = plain.model_hidden(cfg, W, toks)
+    assert len(after) == len(plain.run_order(cfg))
+    dump = str(tmp_path / "hidden")
+    monkeypatch.setenv("CELEG_DUMP_HIDDEN", dump)
+    lm = load_model(folder, dtype="float32", page_tokens=16, n_pages=8, max_requests=2, max_batched_tokens=64)
+    monkeypatch.delenv("CELEG_DUMP_HIDDEN")
+    slot = lm.cache.open()
+    assert lm.cache.prepare(slot, 0, 23)
+    for k, (start, n) in enumerate([(0, 21), (21, 1), (22, 1)]):
+        lm.runner.step([StepEntry(slot, start, toks[start:start + n], [n - 1])])
+        for i in range(len(after)):
+            rows = np.fromfile(os.path.join(dump, f"step{k}_layer{i}.f32"), dtype="<f4").reshape(n, cfg["width"])
+            assert_close_f32(torch.from_numpy(rows), after[i][start:start + n], f"step {k}, entry {i}")
+    lm.close()
+
+
+def test_batches_of_unequal_requests_equal_each_alone(folders):
+    """In 32-bit a row's logits do not depend on what else is in the batch or on how the prompt was
+    cut: every sum of this design runs in an order that the row's own position fixes."""
+    folder = folders("V1", "float32")
+    reqs = requests_of("V1")
+    alone_steps, mixed_steps, cut_steps = whole_schedule(reqs), mixed_schedule(reqs, seed=3), portions_schedule(reqs)
+    lm, _ = load(folder, "float32", alone_steps)
+    alone = EngineDriver(lm).run(alone_steps)
+    for steps in (mixed_steps, cut_steps):
+        lm2, _ = load(folder, "float32", steps)
+        other = EngineDriver(lm2).run(steps)
+        for rid in reqs:
+            assert float((alone[rid] - other[rid]).abs().max()) <= 2e-5 * float(alone[rid].abs().max()), rid
+
+
+def drawn_model(rng):
+    """A configuration drawn at random: widths, head counts and sizes (those the matrix cores take, and
+    others), order and number of layers, windows, kept keys, taps, feed-forwards, the loop and constants."""
+    cfg = {"architecture": "Vabuzen", "vocab": rng.randint(100, 700), "width": rng.choice([64, 96, 160, 192, 200, 320]),
+           "norm": {"eps": rng.choice([1e-6, 1e-5])}}
+    if rng.random() < 0.8:
+        cfg["residual_mult"] = round(rng.uniform(0.3, 1.5), 3)
+    if rng.random() < 0.8:
+        cfg["logit_softcap"] = round(rng.uniform(5.0, 40.0), 2)
+
+    def mlp():
+        r = rng.random()
+        if r < 0.15:
+            return None
+        if r < 0.45:
+            return dense(rng.choice([64, 200, 256]))
+        count = rng.choice([1, 2, 3, 4])
+        per = rng.choice([1, 2, 3, 4])
+        keep = rng.randint(1, count)
+        top = rng.randint(1, min(4, keep * per))
+        return moe(count * per, top, rng.choice([32, 64, 96]), (count, keep) if rng.random() < 0.85 else None,
+                   round(rng.uniform(0.5, 3.0), 2) if rng.random() < 0.8 else None, rng.choice([None, 32, 80, 128]))
+    layers = []
+    n_layers = rng.randint(2, 5)
+    for _ in range(n_layers):
+        if rng.random() < 0.5:
+            kv, dim = rng.choice([1, 2, 3, 4]), rng.choice([16, 32, 48, 64, 80, 128])
+            rot = (rng.choice([100.0, 10000.0, 1e6]), rng.choice([d for d in (4, 16, 32, dim) if d <= dim])) if rng.random() < 0.85 else None
+            mask = (rng.choice([1, 5, 16, 31, 40, 64, 100]), rng.choice([0, 1, 4, 17, 40])) if rng.random() < 0.85 else None
+            layers.append(attention(kv * rng.choice([1, 2, 4]), kv, dim, rng.choice([16, 32, 64, 96, 128]),
+                                    round(dim ** -0.5 * rng.uniform(0.7, 1.5), 4), rng.choice([0, 1, 2, 3, 4, 6]), rot, mask, mlp()))
+        else:
+            dim, rot_dim = rng.choice([16, 32, 48, 64]), rng.choice([0, 8, 16, 32, 64])
+            layers.append(latent(rng.choice([1, 2, 4, 8, 16]), dim, rot_dim, rng.choice([16, 32, 64]), rng.choice([16, 32, 64, 96, 40]),
+                                 round((dim + rot_dim) ** -0.5 * rng.uniform(0.7, 1.5), 4), rng.choice([1000.0, 50000.0]), mlp()))
+    cfg["layers"] = layers
+    if rng.random() < 0.85:
+        start = rng.randint(0, n_layers - 1)
+        cfg["loop"] = {"start": start, "stop": rng.randint(start, n_layers), "times": rng.randint(1, 3)}
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_models_drawn_at_random(tmp_path, seed):
+    """Eight models drawn at random, weights stored in bfloat16, four requests of 20 to 300 tokens,
+    in a mixed schedule and in long and short portions, in 32-bit and in bfloat16."""
+    import random
+    rng = random.Random(2000 + seed)
+    cfg = drawn_model(rng)
+    folder = write_model(tmp_path / "drawn", cfg, seed, torch.bfloat16, std=0.06)
+    c, W = plain.load_model_folder(folder)
+    reqs = {f"r{i}": random_tokens(cfg["vocab"], rng.randint(20, 300), seed=seed * 10 + i) for i in range(4)}
+    ref = {rid: plain.model_logits(c, W, toks) for rid, toks in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        for steps in (mixed_schedule(reqs, seed=seed, decode_tail=rng.randint(3, 20)), portions_schedule(reqs, sizes=(70, 2, 33, 1, 130, 16, 5))):
+            lm, _ = load(folder, dtype, steps)
+            got = EngineDriver(lm).run(steps)
+            for rid in reqs:
+                assert_close(got[rid], ref[rid], dtype, f"drawn model {seed}/{dtype}/{rid}: {json.dumps(cfg)}")
+            lm.close()
+
+
+# ------------------------------------------------------------------ long decoding, pages and slots
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_while_the_windows_pass(folders, dtype):
+    """A short prompt, then 200 tokens one by one (steps replayed from a recorded graph): the windows of
+    50 and 16 keys pass wholly over decoded tokens, their pages go back to the pool but for those of the
+    kept first keys, and the convolutions run from their saved rows alone."""
+    folder = folders("V3", dtype)
+    toks = random_tokens(V3["vocab"], 215, seed=77)
+    steps = tail_decode_schedule({"long": toks}, tail=200)
+    lm, _ = load(folder, dtype, steps)
+    got = EngineDriver(lm).run(steps)["long"]
+    c, W = plain.load_model_folder(folder)
+    assert_close(got, plain.model_logits(c, W, toks), dtype, "long decoding")
+    assert lm.runner.counters()["graph_replays"] > 100
+
+
+def test_pages_of_passed_windows_return_and_kept_ones_stay(folders):
+    """While a request grows, its window groups hold the pages of the window and of the kept first keys
+    only; the group of the compressed rows holds all."""
+    from celeg_amd.engine import StepEntry
+    folder = folders("V1", "float32")
+    toks = random_tokens(V1["vocab"], 200, seed=5)
+    from celeg_amd.engine import load_model
+    lm = load_model(folder, dtype="float32", device=DEV, page_tokens=16, n_pages=16, max_requests=2, max_context=256, max_batched_tokens=256)
+    slot = lm.cache.open()
+    assert lm.cache.prepare(slot, 0, 150)
+    lm.runner.step([StepEntry(slot, 0, toks[:150], [149])])
+    assert lm.cache.prepare(slot, 150, 50)
+    logits = lm.runner.step([StepEntry(slot, 150, toks[150:], list(range(50)))]).detach().cpu()
+    held = sorted(len(p) for p in lm.cache.pages_held(slot))
+    # 13 pages in each of the two groups of compressed rows; windows of 24 and 33 from position 150 on: pages 7 to 12
+    # (positions 127 and 118 lie in page 7), plus page 0 for three kept keys and pages 0 and 1 for twenty
+    assert held == [7, 8, 13, 13], held
+    c, W = plain.load_model_folder(folder)
+    assert_close_f32(logits, plain.model_logits(c, W, toks)[150:], "after the windows passed")
+    lm.cache.close(slot)
+    lm.cache.check()
+
+
+def test_pages_and_slots_used_again(folders):
+    """Ten requests through two slots and a pool of six pages: every page and state slot serves
+    several requests, and each request's logits equal the plain ones (saved rows of a convolution
+    that are not zeroed when their slot is given out again would show at the request's first tokens)."""
+    folder = folders("V1", "float32")
+    reqs = {f"q{i}": random_tokens(V1["vocab"], n, seed=500 + i) for i, n in enumerate([30, 18, 33, 16, 5, 47, 31, 2, 40, 17])}
+    steps = mixed_schedule(reqs, max_live=2, seed=4, decode_tail=6)
+    from celeg_amd.engine import load_model
+    lm = load_model(folder, dtype="float32", device=DEV, page_tokens=16, n_pages=6, max_requests=2, max_context=64,
+                    max_batched_tokens=128)
+    got = EngineDriver(lm).run(steps)
+    c, W = plain.load_model_folder(folder)
+    for rid, toks in reqs.items():
+        assert_close_f32(got[rid], plain.model_logits(c, W, toks), rid)
+    assert all(n == 6 for n in lm.cache.free_pages())
+
+
+# ------------------------------------------------------------------ generation through the entry point
+@pytest.mark.parametrize("name", ["V1", "V2"])
+def test_greedy_generation_through_the_entry_point(folders, name):
+    from celeg_amd.engine import Engine
+    from celeg_amd.sampling import GenerationConfig
+    folder = folders(name, "float32")
+    cfg, W = plain.load_model_folder(folder)
+    prompts = [random_tokens(cfg["vocab"], n, seed=40 + n) for n in (5, 23, 1, 37, 12)]
+    engine = Engine.from_folder(folder, dtype="float32", device=DEV, max_active_requests=3, max_batched_tokens=64,
+                                prefill_chunk_tokens=16, context=128, n_pages=24)
+    greedy = GenerationConfig(temperature=0.0, repetition_penalty=1.0)
+    outs = engine.generate(prompts, max_new_tokens=20, generation=greedy, eos_token_ids=[])
+    for prompt, out in zip(prompts, outs):
+        assert out == plain.greedy(cfg, W, prompt, 20)
+    engine.close()
+
+
+def test_command_line(folders, tmp_path):
+    """``bin/celeg-run`` on a model folder of the design: greedy tokens and the prompt's last logits."""
+    import subprocess
+    import sys
+    import numpy as np
+    folder = folders("V2", "float32")
+    cfg, W = plain.load_model_folder(folder)
+    prompt = random_tokens(cfg["vocab"], 19, seed=5)
+    dump = str(tmp_path / "logits.f32")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "celeg-run"), "--model", folder, "--dtype", "float32", "--prompt",
+                           ",".join(map(str, prompt)), "--max-new-tokens", "8", "--repetition-penalty", "1.0", "--context", "128",
+                           "--runtime-tokens", "--dump-logits", dump], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr
+    line = [l for l in proc.stdout.splitlines() if l.startswith("CELEG_GENERATED_TOKEN_IDS=")][0]
+    assert json.loads(line.split("=", 1)[1]) == plain.greedy(cfg, W, prompt, 8)
+    logits = np.fromfile(dump, dtype="<f4")
+    assert_close_f32(torch.from_numpy(logits.copy()), plain.model_logits(cfg, W, prompt)[-1], "command line")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_program(folders, tmp_path, dtype):
+    """``bin/trace_run`` in a process of its own: four schedules one after the other, a pool sized for
+    the live requests only, logits read from the files it writes."""
+    from helpers import TraceClient
+    folder = folders("V1", dtype)
+    reqs = requests_of("V1")
+    ref = plain_logits(folder, ("V1", dtype), reqs)
+    all_steps = []
+    for tag, make in (("w", whole_schedule), ("t", tail_decode_schedule), ("p", portions_schedule), ("m", mixed_schedule)):
+        for s in make({f"{tag}{rid}": toks for rid, toks in reqs.items()}):
+            all_steps.append(dict(s, step=len(all_steps)))
+    client = TraceClient(folder, dtype, str(tmp_path), peak_tokens(all_steps))
+    got = {}
+    for s in all_steps:
+        logits = client.step(s["step"], s["entries"], s["end"])
+        row = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got.setdefault(e["id"], []).append(torch.as_tensor(logits[row]))
+                row += 1
+    assert client.close() == 0
+    for rid_tagged, rows in got.items():
+        assert_close(torch.stack(rows), ref[rid_tagged[1:]], dtype, f"trace/{dtype}/{rid_tagged}")
+
+
+# ------------------------------------------------------------------ each mechanism alone
+def alone_architectures():
+    """"VabuzenPartsAlone": one block whose sub-layers read the stream as it is (x + mixer(x) + ff(x)).
+    "VabuzenBlockAlone": one block of dynamic tanh norms before and after each sub-layer, with the layer's
+    factor.  The embedding table is the input (tokens 0..T-1), the head gives the stream's rows back."""
+    from celeg_amd.config import LayerSpec, ModelSpec, PartSpec, RunStep, register_architecture, registered_architectures
+    if "VabuzenPartsAlone" in registered_architectures():
+        return
+
+    def parts(cfg, shapes):
+        W, rows = cfg["width"], cfg["rows"]
+        part = lambda key, neutral: PartSpec.from_json(cfg[key]) if cfg.get(key) else neutral
+        block = LayerSpec(part("mixer", PartSpec("none", {"width": W})), PartSpec("identity"), part("ffn", PartSpec("none")),
+                          PartSpec("identity"), "parallel")
+        return ModelSpec("VabuzenPartsAlone", rows, W, 512, PartSpec("embedding", {"vocab": rows, "width": W}, {"table": "table"}),
+                         (block,), (RunStep(0, None, False),), PartSpec("identity"), PartSpec("hidden", {"width": W}))
+
+    def block(cfg, shapes):
+        W, rows = cfg["width"], cfg["rows"]
+        norm = lambda name: PartSpec("dynamic_tanh", {"width": W, "bias": True}, {"weight": name, "alpha": name + ".alpha", "bias": name + ".b"})
+        layer = LayerSpec(PartSpec.from_json(cfg["mixer"]), norm("n1"), PartSpec.from_json(cfg["ffn"]), norm("n2"), "sandwich_norm",
+                          mixer_post_norm=norm("n1b"), ffn_post_norm=norm("n2b"), residual_scale=cfg["factor"])
+        return ModelSpec("VabuzenBlockAlone", rows, W, 512, PartSpec("embedding", {"vocab": rows, "width": W}, {"table": "table"}),
+                         (layer,), (RunStep(0, None, False),), PartSpec("identity"), PartSpec("hidden", {"width": W}))
+    register_architecture("VabuzenPartsAlone", parts)
+    register_architecture("VabuzenBlockAlone", block)
+
+
+CUT = (5, 2, 9, 1, 3, 17)
+
+
+def run_alone(tmp_path, cfg, tensors, cut=CUT, dtype="float32", knobs=None, n_pages=8, architecture="VabuzenPartsAlone"):
+    """What the block makes of rows 0..T-1 (the tensor "table"), in portions."""
+    from celeg_amd.engine import load_model
+    from celeg_amd.weights.safetensors_io import write_safetensors
+    alone_architectures()
+    cfg = dict(cfg, architectures=[architecture])
+    os.makedirs(tmp_path, exist_ok=True)
+    with open(os.path.join(tmp_path, "config.json"), "w") as fh:
+        json.dump(cfg, fh)
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    write_safetensors(os.path.join(tmp_path, "model.safetensors"), {k: v.to(storage).contiguous() for k, v in tensors.items()})
+    steps = portions_schedule({"x": list(range(cfg["rows"]))}, sizes=cut)
+    lm = load_model(str(tmp_path), dtype=dtype, device=DEV, page_tokens=16, n_pages=n_pages, max_requests=2, max_context=16 * n_pages,
+                    max_batched_tokens=max(64, max(cut)))
+    for k, v in (knobs or {}).items():
+        lm.set_knob(k, v)
+    return EngineDriver(lm).run(steps)["x"].double(), lm
+
+
+def attention_case(T, W_, H, G, D, V, scale, taps=3, rot=None, mask=None, seed=1, x_std=1.0, sink=True):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)
+    t = {"table": r(T, W_) * x_std, "q": r(H * D, W_) * 0.3, "k": r(G * D, W_) * 0.3, "v": r(G * V, W_) * 0.3, "o": r(W_, H * V) * 0.3}
+    names = {"q": "q", "k": "k", "v": "v", "o": "o"}
+    params = {"width": W_, "heads": H, "kv_heads": G, "head_dim": D, "v_dim": V, "scale": scale, "sink_one": sink, "taps": taps}
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": V, "scale": scale}
+    if taps:
+        m["conv"] = taps
+        for c, n in (("q", H * D), ("k", G * D), ("v", G * V)):
+            t[c + ".conv"] = r(n, taps) * 0.6
+            names[c + "_conv"] = c + ".conv"
+    if rot:
+        m["rot"] = {"base": rot[0], "dims": rot[1]}
+        params["position"] = {"kind": "rope", "params": {"theta": rot[0], "rotary_dim": rot[1], "head_dim": D, "pairing": "neighbours"}}
+    if mask:
+        m["mask"] = {"size": mask[0], "keep_first": mask[1]}
+        params["window"], params["keep_first"] = mask
+    return t, m, {"kind": "biased_attention", "params": params, "tensors": names}
+
+
+def doubles(t):
+    return {k: v.double() for k, v in t.items()}
+
+
+@pytest.mark.parametrize("taps,rot,mask", [(3, (100.0, 12), (9, 2)), (0, None, None), (1, (10000.0, 4), (16, 0)), (6, (50.0, 8), (1, 3)),
+                                           (4, None, (17, 20)), (2, (1000.0, 2), None)])
+def test_window_attention_alone(tmp_path, taps, rot, mask):
+    T, W_ = 45, 40
+    t, m, part = attention_case(T, W_, 6, 3, 12, 20, 0.3, taps, rot, mask)
+    got, _ = run_alone(tmp_path, {"width": W_, "rows": T, "mixer": part}, t)
+    Wd = doubles(t)
+    assert_close_f32(got, Wd["table"] + plain.window_attention(Wd["table"], Wd, "", m), "attention behind convolutions alone")
+
+
+def test_the_one_in_the_denominator_the_pairing_and_the_taps_show():
+    """The plain attention with an ordinary softmax, with the halves paired instead of neighbours, with
+    the taps in reverse order or with a window or a number of kept keys that is one off differs by far
+    more than any tolerance."""
+    t, m, _ = attention_case(60, 24, 2, 1, 16, 16, 0.5, 3, (100.0, 16), (9, 3))
+    Wd = doubles(t)
+    right = plain.window_attention(Wd["table"], Wd, "", m)
+
+    def moved(out):
+        return float((out - right).abs().max()) / float(right.abs().max())
+    n = 60
+    H, D = 2, 16
+    # an ordinary softmax: the same scores, weights that sum to one
+    q, k, v = (plain.causal_taps(Wd["table"] @ Wd[c].T, Wd[c + ".conv"]) for c in "qkv")
+    pos = torch.arange(n)
+    qh, kh = plain.rotate_neighbours(q.view(n, H, D), pos, 100.0, 16), plain.rotate_neighbours(k.view(n, 1, D), pos, 100.0, 16)
+    out = torch.zeros(n, H, D, dtype=torch.float64)
+    for i in range(n):
+        seen = [j for j in range(i + 1) if i - j < 9 or j < 3]
+        for a in range(H):
+            out[i, a] = torch.softmax((kh[seen, 0] @ qh[i, a]) * 0.5, 0) @ v.view(n, 1, D)[seen, 0]
+    assert moved(out.reshape(n, H * D) @ Wd["o"].T) > 0.1
+    flipped = dict(Wd, **{c + ".conv": Wd[c + ".conv"].flip(1) for c in "qkv"})
+    assert moved(plain.window_attention(Wd["table"], flipped, "", m)) > 0.1
+    for size, keep in ((8, 3), (10, 3), (9, 2), (9, 4)):
+        assert moved(plain.window_attention(Wd["table"], Wd, "", dict(m, mask={"size": size, "keep_first": keep}))) > 0.02, (size, keep)
+    halves = plain.rotate_halves(q.view(n, H, D), pos, 100.0, 16)
+    assert float((halves - qh).abs().max()) > 0.1 * float(qh.abs().max())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_keys_at_the_windows_edge_and_kept_first_keys(tmp_path, dtype):
+    """Rows whose weight sits on one key: the last key inside a window of 40 and the first one outside, the
+    last kept first key (position 4 of 5) hundreds of positions back and the first one not kept, for rows
+    inside a prompt's portion and rows decoded alone.  Queries and keys are the same map of the input's first
+    half, in which the marked rows point one way and are long, so a querying row's score against a marked key
+    is far above all others; the marked rows differ in the input's second half, which only the values read.
+    No convolution or rotation blurs them.  The plain result with a window or a number of kept keys that is
+    one off differs in these rows by more than a tenth."""
+    T, W_, H, D = 300, 32, 2, 32
+    size, keep = 40, 5
+    t, m, part = attention_case(T, W_, H, H, D, D, 0.25, 0, None, (size, keep), seed=5, x_std=0.3)
+    t["q"][:, W_ // 2:] = 0.0
+    t["k"] = t["q"].clone()
+    g = torch.Generator().manual_seed(9)
+    direction = torch.randn(W_, generator=g)
+    direction[W_ // 2:] = 0.0
+    direction = direction / direction.norm()
+    # marked keys: 4 (kept) and 5 (not), and for the query rows 200 (in a portion) and 290 (decoded) the keys at
+    # distance size - 1 (inside) and size (outside)
+    queries = (200, 290)
+    for row in (4, 5) + tuple(q - size + 1 for q in queries) + tuple(q - size for q in queries):
+        own = torch.randn(W_, generator=g)
+        own[:W_ // 2] = 0.0
+        t["table"][row] = 8.0 * direction + 6.0 * own / own.norm()
+    for row in queries:
+        t["table"][row] = 2.0 * direction
+    Wd = doubles(t)
+    want = Wd["table"] + plain.window_attention(Wd["table"], Wd, "", m)
+    for other in ({"size": size + 1, "keep_first": keep}, {"size": size - 1, "keep_first": keep}, {"size": size, "keep_first": keep + 1},
+                  {"size": size, "keep_first": keep - 1}):
+        off = Wd["table"] + plain.window_attention(Wd["table"], Wd, "", dict(m, mask=other))
+        for row in queries:
+            assert float((want[row] - off[row]).abs().max()) > 0.1 * float(want[row].abs().max()), (other, row)
+    cut = (130, 2, 97, 31, 16, 1, 7) + (1,) * 16
+    got, lm = run_alone(tmp_path, {"width": W_, "rows": T, "mixer": part}, t, cut=cut, dtype=dtype, n_pages=20)
+    if dtype == "float32":
+        assert_close_f32(got, want, "keys at the edges")
+    else:
+        Wb = {k_: v.bfloat16().double() for k_, v in Wd.items()}
+        ref = Wb["table"] + plain.window_attention(Wb["table"], Wb, "", m)
+        for row in queries + (120, 299):
+            assert float((got[row] - ref[row]).abs().max()) <= 0.03 * float(ref[row].abs().max()), row
+        assert lm.paths()["attention_biased_rows"] > 0 and lm.paths()["attention_biased_decode"] > 0
+
+
+@pytest.mark.parametrize("D,V", [(32, 32), (64, 128), (96, 64), (128, 96)])
+def test_matrix_core_attention_equals_the_general_kernel(tmp_path, D, V):
+    """bfloat16: the kernels on the matrix cores against the kernel that scores key by key, on the same
+    pages, with windows and kept first keys that end before, at and behind the borders of pages and of the
+    blocks of 64 keys (kept keys that the window still covers, that fill more than a block, none), in whole
+    prompts, portions and single tokens.  The two differ in the rounding of the weights to bfloat16 only."""
+    T, W_ = 300, 64
+    for mask in ((7, 3), (64, 64), (65, 1), (16, 70), (40, 0), (200, 9), None):
+        t, m, part = attention_case(T, W_, 4, 2, D, V, D ** -0.5, 3, (10000.0, D // 2), mask, seed=D + V, x_std=1.5)
+        got = {}
+        long_cut = (15, 2, 17, 1, 130, 3, 16, 64)
+        for form, cut in (("general", long_cut), (-1, long_cut), (0, long_cut), (1, long_cut), (-1, (300,)), (-1, (270,) + (1,) * 30)):
+            knobs = {"use_biased_mfma": 0} if form == "general" else {"biased_rows_form": form}
+            out, lm = run_alone(tmp_path / f"{mask}_{form}_{len(cut)}", {"width": W_, "rows": T, "mixer": part}, t, cut=cut, dtype="bfloat16",
+                                knobs=knobs, n_pages=20)
+            took = lm.paths()["attention_biased_rows"] + lm.paths()["attention_biased_decode"]
+            assert (took > 0) == (form != "general")
+            got[(form, len(cut))] = out
+        ref = got[("general", 8)]
+        for key, out in got.items():
+            rel = float((out - ref).pow(2).mean().sqrt() / ref.pow(2).mean().sqrt())
+            assert rel <= 1e-2, f"heads of {D} and {V}, mask {mask}, form {key}: rel rms {rel:.3e}"
+
+
+def latent_case(T, W_, H, D, R, V, rank, scale, base, seed=3, x_std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)
+    t = {"table": r(T, W_) * x_std, "q": r(H * (D + R), W_) * 0.3, "dkv": r(rank + R, W_) * 0.3, "dkv.norm": 1 + 0.3 * r(rank),
+         "uk": r(H * D, rank) * 0.4, "uv": r(H * V, rank) * 0.4, "o": r(W_, H * V) * 0.3}
+    names = {"q": "q", "dkv": "dkv", "dkv_norm": "dkv.norm", "uk": "uk", "uv": "uv", "o": "o"}
+    params = {"width": W_, "heads": H, "dim": D, "rot_dim": R, "vdim": V, "kv_rank": rank, "scale": scale, "eps": 1e-5, "sink": False, "gate": False}
+    m = {"heads": H, "dim": D, "rot_dim": R, "vdim": V, "kv_rank": rank, "scale": scale}
+    if R:
+        m["rot"] = {"base": base, "dims": R}
+        params["position"] = {"kind": "rope", "params": {"theta": base, "rotary_dim": R, "head_dim": R, "pairing": "halves"}}
+    return t, m, {"kind": "latent_attention", "params": params, "tensors": names}
+
+
+@pytest.mark.parametrize("H,D,R,V,rank", [(5, 12, 8, 14, 20), (2, 8, 0, 8, 12), (16, 32, 16, 32, 64), (1, 16, 32, 24, 48)])
+def test_latent_attention_with_split_halves_alone(tmp_path, H, D, R, V, rank):
+    T, W_ = 45, 40
+    t, m, part = latent_case(T, W_, H, D, R, V, rank, (D + R) ** -0.5, 300.0)
+    Wd = doubles(t)
+    want = Wd["table"] + plain.compressed_attention(Wd["table"], Wd, "", m, 1e-5)
+    got, lm = run_alone(tmp_path, {"width": W_, "rows": T, "mixer": part}, t)
+    assert_close_f32(got, want, "latent attention alone")
+    assert lm.paths()["attention_latent"] > 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_compressed_row_far_back_among_hundreds(tmp_path, dtype):
+    """A compressed row is normed, so no key is long; the queries are.  W_uk maps the compressed row as minus W_q
+    maps the input, row 3's input points against those of rows 250 (inside a prompt's portion) and 299 (decoded
+    alone), and these are long: those rows' weight sits on a key 247 and 296 positions back, over a dozen and a
+    half pages (their own key scores lowest of all); left out, the rows' outputs are others."""
+    T, W_, H, D, R, V, rank = 300, 32, 16, 32, 16, 32, 64
+    t, m, part = latent_case(T, W_, H, D, R, V, rank, 0.2, 1e6, seed=7, x_std=0.3)
+    direction = torch.randn(W_, generator=torch.Generator().manual_seed(9))
+    direction = direction / direction.norm()
+    for row, length in ((3, -1.0), (250, 6.0), (299, 6.0)):
+        t["table"][row] = length * direction
+    # a head's plain key of row j is W_uk c_j: uk = -(q's plain rows) pinv(dkv's first rows)
+    down = t["dkv"][:rank].double()
+    qp = t["q"].double().view(H, D + R, W_)[:, :D].reshape(H * D, W_)
+    t["uk"] = -(qp @ torch.linalg.pinv(down)).float()
+    Wd = doubles(t)
+    want = Wd["table"] + plain.compressed_attention(Wd["table"], Wd, "", m, 1e-5)
+    without = Wd["table"].clone()
+    without[3] = Wd["table"][4]
+    lost = without + plain.compressed_attention(without, Wd, "", m, 1e-5)
+    for row in (250, 299):
+        assert float((want[row] - lost[row]).abs().max()) > 0.1 * float(want[row].abs().max())
+    cut = (130, 2, 97, 31, 16, 1, 7, 3, 2) + (1,) * 11
+    got, lm = run_alone(tmp_path, {"width": W_, "rows": T, "mixer": part}, t, cut=cut, dtype=dtype, n_pages=20)
+    if dtype == "float32":
+        assert_close_f32(got, want, "a far compressed row")
+    else:
+        Wb = {k_: v.bfloat16().double() for k_, v in Wd.items()}
+        ref = Wb["table"] + plain.compressed_attention(Wb["table"], Wb, "", m, 1e-5)
+        for row in (250, 299, 120):
+            assert float((got[row] - ref[row]).abs().max()) <= 0.05 * float(ref[row].abs().max()), row
+        assert lm.paths()["attention_latent_rows"] > 0 and lm.paths()["attention_latent_decode"] > 0
+
+
+def experts_case(T, W_, ff, experts, top, groups, scale, shared, seed=5):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g)
+    t = {"table": r(T, W_), "router": r(experts, W_) * 0.5}
+    names = {"router": "router"}
+    for e in range(experts):
+        for what, shape in (("gate", (ff, W_)), ("up", (ff, W_)), ("down", (W_, ff))):
+            t[f"e{e}.{what}"] = r(*shape) * 0.3
+            names[f"{what}.{e}"] = f"e{e}.{what}"
+    params = {"width": W_, "ff": ff, "experts": experts, "top": top, "score": "sigmoid", "renormalize": True, "renormalize_eps": 1e-20,
+              "route_scale": scale, "weight_on": "output"}
+    f = {"router": {"experts": experts, "top": top, "scale": scale}}
+    if groups:
+        params["groups"] = {"count": groups[0], "keep": groups[1]}
+        f["router"]["groups"] = params["groups"]
+    if shared:
+        for what, shape in (("gate", (shared, W_)), ("up", (shared, W_)), ("down", (W_, shared))):
+            t[f"shared.{what}"] = r(*shape) * 0.3
+            names[f"shared.{what}"] = f"shared.{what}"
+        params["shared"] = {"kind": "swiglu", "params": {"width": W_, "ff": shared}}
+        f["shared"] = {"ff": shared}
+    return t, f, {"kind": "routed_experts", "params": params, "tensors": names}
+
+
+@pytest.mark.parametrize("experts,top,groups,scale,shared", [(12, 3, (4, 2), 2.0, 40), (5, 2, None, 1.0, None), (8, 1, (8, 3), 0.5, 16),
+                                                             (6, 6, (2, 2), 1.5, 24), (9, 2, (3, 1), 3.0, None), (70, 4, (7, 2), 1.0, 8)])
+def test_routed_experts_in_groups_alone(tmp_path, experts, top, groups, scale, shared):
+    T, W_, ff = 33, 40, 24
+    t, f, part = experts_case(T, W_, ff, experts, top, groups, scale, shared)
+    got, lm = run_alone(tmp_path, {"width": W_, "rows": T, "ffn": part}, t)
+    Wd = doubles(t)
+    assert_close_f32(got, Wd["table"] + plain.routed_ff(Wd["table"], Wd, "", f), "routed experts alone")
+    assert lm.paths()["routed_experts"] > 0
+
+
+def test_the_groups_the_renormalization_and_the_shared_expert_show():
+    """Without the groups other experts are chosen for many rows (the largest scores of a row often lie in a
+    group that loses); weights not divided by their sum, a factor left out or the shared expert left out move
+    the output by tens of percent."""
+    t, f, _ = experts_case(64, 40, 24, 12, 3, (4, 2), 2.0, 40)
+    Wd = doubles(t)
+    right = plain.routed_ff(Wd["table"], Wd, "", f)
+    score = torch.sigmoid(Wd["table"] @ Wd["router"].T)
+    differ = sum(sorted(plain.choose_experts(score[i], f["router"])[0]) != sorted(plain.choose_experts(score[i], {"experts": 12, "top": 3})[0])
+                 for i in range(64))
+    assert differ >= 16
+    moved = lambda out: float((out - right).abs().max()) / float(right.abs().max())
+    assert moved(plain.routed_ff(Wd["table"], Wd, "", dict(f, router=dict(f["router"], scale=1.0)))) > 0.1
+    assert moved(plain.routed_ff(Wd["table"], Wd, "", dict(f, shared=None))) > 0.1
+    assert moved(plain.routed_ff(Wd["table"], Wd, "", dict(f, router=dict(f["router"], groups={"count": 4, "keep": 1})))) > 0.1
+
+
+def test_dense_feed_forward_alone(tmp_path):
+    torch.manual_seed(4)
+    T, W_, ff = 29, 36, 50
+    t = {"table": torch.randn(T, W_) * 2, "up": torch.randn(ff, W_) * 0.3, "up.b": torch.randn(ff), "down": torch.randn(W_, ff) * 0.3,
+         "down.b": torch.randn(W_)}
+    part = {"kind": "mlp", "params": {"width": W_, "ff": ff, "activation": "gelu_tanh", "bias": True},
+            "tensors": {"up": "up", "up_bias": "up.b", "down": "down", "down_bias": "down.b"}}
+    got, _ = run_alone(tmp_path, {"width": W_, "rows": T, "ffn": part}, t)
+    Wd = doubles(t)
+    assert_close_f32(got, Wd["table"] + plain.dense_ff(Wd["table"], Wd, ""), "dense feed-forward alone")
+
+
+@pytest.mark.parametrize("factor,W_", [(0.5, 36), (1.0, 40), (1.7, 1100), (0.25, 2100)])
+def test_block_of_dynamic_tanh_norms_alone(tmp_path, factor, W_):
+    """x <- x + m post(mixer(pre(x))), then the same around the feed-forward, every norm tanh(alpha x) w + b
+    with an alpha, weight and bias of its own; rows of several widths (up to 1,024 and 2,048 values a thread
+    holds its share of a row in registers, above the row lies in LDS)."""
+    torch.manual_seed(6)
+    T, ff = 21, 24
+    t = {"table": torch.randn(T, W_) * 2, "up": torch.randn(ff, W_) * 0.1, "up.b": torch.randn(ff), "down": torch.randn(W_, ff) * 0.3,
+         "down.b": torch.randn(W_)}
+    at, am, apart = attention_case(T, W_, 2, 1, 8, 8, 0.3, 2, (100.0, 4), (6, 2), seed=3)
+    for k, v in at.items():
+        if k != "table":
+            t["a." + k] = v * (0.3 if k in "qkvo" else 1.0)
+    apart = dict(apart, tensors={k: "a." + v for k, v in apart["tensors"].items()})
+    for n in ("n1", "n1b", "n2", "n2b"):
+        t[n], t[n + ".b"], t[n + ".alpha"] = 1 + 0.3 * torch.randn(W_), torch.randn(W_), torch.tensor(0.3 + torch.rand(()).item())
+    ffn = {"kind": "mlp", "params": {"width": W_, "ff": ff, "activation": "gelu_tanh", "bias": True},
+           "tensors": {"up": "up", "up_bias": "up.b", "down": "down", "down_bias": "down.b"}}
+    got, _ = run_alone(tmp_path, {"width": W_, "rows": T, "mixer": apart, "ffn": ffn, "factor": factor}, t, architecture="VabuzenBlockAlone",
+                       cut=(5, 2, 9, 1, 4))
+    Wd = doubles(t)
+    x = Wd["table"]
+    x = x + factor * plain.dynamic_tanh(plain.window_attention(plain.dynamic_tanh(x, Wd, "n1"), Wd, "a.", am), Wd, "n1b")
+    x = x + factor * plain.dynamic_tanh(plain.dense_ff(plain.dynamic_tanh(x, Wd, "n2"), Wd, ""), Wd, "n2b")
+    assert_close_f32(got, x, "block of dynamic tanh norms alone")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_saved_rows_of_the_convolutions_between_steps(tmp_path, dtype):
+    """Taps of six and weights that put most on the oldest inputs: a token's q, k and v hang on the five
+    tokens before it, which lie in an earlier step for the first rows of every portion (and for every single
+    token), in portions shorter than the taps too.  A model whose saved rows are lost, zeroed or taken from
+    another slot gives other logits; two requests run side by side."""
+    cfg = {"architecture": "Vabuzen", "vocab": 140, "width": 64, "norm": {"eps": 1e-5}, "residual_mult": 1.0,
+           "layers": [attention(4, 2, 16, 16, 0.25, 6, (100.0, 8), (30, 2), dense(32)), attention(2, 2, 32, 32, 0.2, 6, None, None, None)]}
+    old = lambda w: w * torch.tensor([3.0, 2.0, 1.0, 0.3, 0.2, 0.1])
+    storage = torch.float32 if dtype == "float32" else torch.bfloat16
+    folder = write_model(tmp_path / "conv", cfg, 7, storage, std=0.1,
+                         change={f"l{i}.mix.{c}.conv": old for i in (0, 1) for c in "qkv"})
+    c, W = plain.load_model_folder(folder)
+    reqs = {"a": random_tokens(cfg["vocab"], 120, seed=3), "b": random_tokens(cfg["vocab"], 90, seed=4)}
+    ref = {rid: plain.model_logits(c, W, toks) for rid, toks in reqs.items()}
+    # the old inputs matter: with the newest tap alone the logits are others
+    newest = {k: (v * torch.tensor([0.0, 0.0, 0.0, 0.0, 0.0, 1.0]).double() if k.endswith(".conv") else v) for k, v in W.items()}
+    assert float((plain.model_logits(c, newest, reqs["a"]) - ref["a"]).abs().max()) > 0.1 * float(ref["a"].abs().max())
+    for steps in (tail_decode_schedule(reqs, tail=30), portions_schedule(reqs, sizes=(37, 2, 3, 1, 4, 5, 2, 16, 1, 31)),
+                  mixed_schedule(reqs, seed=5, decode_tail=10)):
+        lm, _ = load(folder, dtype, steps)
+        got = EngineDriver(lm).run(steps)
+        for rid in reqs:
+            assert_close(got[rid], ref[rid], dtype, f"saved rows/{dtype}/{rid}")
