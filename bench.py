@@ -197,6 +197,32 @@ KIVORAX_SHAPES = {
            kifetar_beside(2048, KIVORAX_PATTERN, 16, 8, 128, 16, 8, 128, 128, 4096)),
 }
 
+# Vabuzen beside Regipel, the closest existing design (attention over compressed rows, routed experts, a looped
+# range of layers): six layers of which the second and third run twice, so eight runs; windowed attention behind
+# short convolutions in the first and fourth layer, attention over compressed rows in the others; dense and routed
+# feed-forwards in turn.  Regipel beside it has one residual stream, eight layers of the same compressed attention and
+# in every layer as many experts a token as Vabuzen's chosen and shared ones together.
+def vabuzen_shape(width, heads, kv_heads, dim, window, l_dim, l_rot, rank, experts, top, groups, ff, shared, dense_ff, vocab=65536):
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "conv": 4,
+                 "rot": {"base": 10000.0, "dims": dim}, "mask": {"size": window, "keep_first": 4}}
+    latent = {"heads": heads, "dim": l_dim, "rot_dim": l_rot, "vdim": l_dim, "kv_rank": rank, "scale": (l_dim + l_rot) ** -0.5,
+              "rot": {"base": 500000.0, "dims": l_rot}}
+    moe = {"kind": "moe", "expert": {"ff": ff}, "shared": {"ff": shared},
+           "router": {"experts": experts, "top": top, "scale": 2.5, "groups": {"count": groups[0], "keep": groups[1]}}}
+    dense = {"kind": "dense", "ff": dense_ff}
+    kinds = {"a": ("attention", attention), "l": ("latent_attention", latent)}
+    layers = [{"type": kinds[c][0], "mixer": kinds[c][1], "mlp": moe if i % 2 else dense} for i, c in enumerate("allall")]
+    return {"architecture": "Vabuzen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.5, "logit_softcap": 30.0,
+            "loop": {"start": 1, "stop": 3, "times": 2}, "max_context": 8192, "layers": layers}
+
+
+VABUZEN_SHAPES = {
+    "1k": (vabuzen_shape(1024, 16, 8, 64, 1024, 64, 32, 256, 16, 2, (4, 2), 1024, 1024, 3072),
+           regipel_shape(1024, 8, 16, 64, 32, 64, 256, 16, 3, 1024, streams=None)),
+    "2k": (vabuzen_shape(2048, 16, 8, 128, 1024, 128, 64, 512, 32, 4, (8, 4), 1024, 2048, 6144),
+           regipel_shape(2048, 8, 16, 128, 64, 128, 512, 32, 6, 1024, streams=None)),
+}
+
 DESIGN_SHAPES = {
     "1k": (regipel_shape(1024, 8, 16, 64, 32, 64, 256, 16, 2, 1024), lfm2_shape(1024, 16, 8, 2048, set(range(8)), 8, 8192)),
     "2k": (regipel_shape(2048, 8, 16, 128, 64, 128, 512, 32, 4, 1024), lfm2_shape(2048, 32, 8, 4096, set(range(8)), 8, 8192)),
@@ -213,7 +239,7 @@ def design(shapes, steps: int, warmup: int, batch: int, layers: int = 0, profile
     out = {}
     for shape in shapes:
         table, beside = {"kifetar": (KIFETAR_SHAPES, "lfm2_hybrid"), "kivorax": (KIVORAX_SHAPES, "kifetar_beside"),
-                         "regipel": (DESIGN_SHAPES, "lfm2_attention")}[which]
+                         "regipel": (DESIGN_SHAPES, "lfm2_attention"), "vabuzen": (VABUZEN_SHAPES, "regipel_beside")}[which]
         for label, cfg in zip((which, beside), table[shape]):
             if profile_only and label != profile_only:
                 continue
@@ -244,7 +270,8 @@ def design(shapes, steps: int, warmup: int, batch: int, layers: int = 0, profile
                 "layers": len(lm.native.info["spec"]["order"])}
             engine.close()
     title = {"kifetar": "Kifetar beside LFM2 convolution and attention layers", "regipel": "Regipel beside LFM2 attention layers",
-             "kivorax": "Kivorax beside Kifetar attention and delta-rule layers"}[which]
+             "kivorax": "Kivorax beside Kifetar attention and delta-rule layers",
+             "vabuzen": "Vabuzen beside Regipel layers of one residual stream"}[which]
     print(json.dumps({"metric": title + " at equal size: prefill tok/s @ 2048 tokens, "
                                 f"decode tok/s @ batch {batch}, context 2048 (bf16, random weights)",
                       "phase": "design", "design": which, "batch": batch, "steps": steps, "warmup": warmup, "dtype": "bf16",
@@ -274,9 +301,9 @@ def main() -> int:
                          "(default 2048, the headline's); with --phase prefill: tokens of the same "
                          "prompt that the cache holds before the measured portion of 2,048 (default 0)")
     ap.add_argument("--design-shape", default="1k,2k", help="with --phase design: which sizes (1k, 2k)")
-    ap.add_argument("--design", default="regipel", choices=["regipel", "kifetar", "kivorax"],
+    ap.add_argument("--design", default="regipel", choices=["regipel", "kifetar", "kivorax", "vabuzen"],
                     help="with --phase design: which design is measured beside its closest LFM2 shape")
-    ap.add_argument("--design-model", default="", choices=["", "regipel", "lfm2_attention", "kifetar", "lfm2_hybrid", "kivorax", "kifetar_beside"],
+    ap.add_argument("--design-model", default="", choices=["", "regipel", "lfm2_attention", "kifetar", "lfm2_hybrid", "kivorax", "kifetar_beside", "vabuzen", "regipel_beside"],
                     help="with --phase design: only this model (for profiling)")
     ap.add_argument("--phase", choices=["all", "prefill", "decode", "serve", "design"], default="all",
                     help="for profiling: run only the prefill measurement, or only the batch-8 "

@@ -103,8 +103,14 @@ V3 = {"architecture": "Vabuzen", "vocab": 260, "width": 128, "norm": {"eps": 1e-
       "layers": [attention(2, 1, 128, 96, 0.09, 2, (500000.0, 32), (50, 18), moe(9, 2, 48, (3, 3), 1.0, 64)),
                  latent(8, 32, 32, 32, 64, 0.125, 10000.0, dense(64)),
                  attention(4, 2, 96, 128, 0.1, 4, (10000.0, 96), (16, 1), dense(96))]}
-MODELS = {"V1": (V1, 41), "V2": (V2, 42), "V3": (V3, 43)}
-LENGTHS = {"V1": [40, 57, 90, 128, 65, 33], "V2": [45, 130, 64, 100, 17, 33], "V3": [31, 32, 150, 64, 49, 80]}
+# sizes that are multiples of two only: width, vocabulary, heads, ranks and feed-forwards that fill no tile or vector load
+V4 = {"architecture": "Vabuzen", "vocab": 333, "width": 100, "norm": {"eps": 1e-6}, "residual_mult": 0.5, "logit_softcap": 15.0,
+      "loop": {"start": 1, "stop": 2, "times": 2},
+      "layers": [attention(3, 1, 20, 12, 0.22, 3, (10000.0, 10), (11, 2), dense(50)),
+                 latent(3, 10, 6, 14, 18, 0.25, 777.0, moe(6, 2, 20, (3, 2), 2.0, 30)),
+                 latent(7, 6, 2, 6, 10, 0.35, 100.0, dense(34))]}
+MODELS = {"V1": (V1, 41), "V2": (V2, 42), "V3": (V3, 43), "V4": (V4, 44)}
+LENGTHS = {"V1": [40, 57, 90, 128, 65, 33], "V2": [45, 130, 64, 100, 17, 33], "V3": [31, 32, 150, 64, 49, 80], "V4": [70, 19, 101, 64, 13, 50]}
 SCHEDULES = {"whole": whole_schedule, "tail12": lambda reqs: tail_decode_schedule(reqs, tail=12),
              "portions": portions_schedule, "mixed": mixed_schedule}
 
@@ -190,7 +196,7 @@ def test_engine_matches_plain(folders, name, dtype, mode):
     assert lm.cache.n_free_slots == 4 and lm.cache.free_pages() == [max_tokens // 16] * len(lm.cache.free_pages())
     paths = lm.paths()
     assert paths["attention_biased"] > 0 and paths["attention_latent"] > 0 and paths["routed_experts"] > 0
-    if dtype == "bfloat16" and name != "V2":
+    if dtype == "bfloat16" and name in ("V1", "V3"):
         assert paths["attention_biased_rows"] + paths["attention_biased_decode"] > 0     # the matrix cores took these heads
 
 
