@@ -79,41 +79,41 @@ __global__ __launch_bounds__(CELEG_WAVE) void biased_attention_kernel(
     // the kept first keys that the window has passed, then the window (or everything)
     const int kept = min(keep_first, first);
     for (int phase = kept > 0 ? 0 : 1; phase < 2; ++phase) {
-    const int lo = phase == 0 ? 0 : first, hi = phase == 0 ? kept - 1 : pos;
-    for (int base = lo; base <= hi; base += CELEG_WAVE) {
-        const int key = base + lane;
-        float score = -INFINITY;
-        if (key <= hi) {
-            const T* kp = k_pool + ba_k_offset(pages[key / page_tokens], n_layers, layer, kv_heads, kvh, page_tokens,
-                                               key % page_tokens, head_dim);
-            float dot = 0.f;
-            for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(kp[d]), dot);
-            score = dot * s;
-            if (r1) score -= b1 * logf(1.0f + b2 * static_cast<float>(pos - key));
-        }
-        const float new_top = fmaxf(top, wave_max(score));     // (the round holds at least one visible key)
-        const float p = key <= hi ? expf(score - new_top) : 0.f;
-        const float keep = expf(top - new_top);                // 0 in the first round
-        total = total * keep + wave_sum(p);
-        top = new_top;
-        ps[lane] = p;
-        __syncthreads();
-        const int n_keys = min(CELEG_WAVE, hi - base + 1);
-#pragma unroll
-        for (int j = 0; j < BA_MAX_V_CHUNKS; ++j) acc[j] *= keep;
-        for (int kk = 0; kk < n_keys; ++kk) {
-            const int key2 = base + kk;
-            const T* vp = v_pool + ba_v_offset(pages[key2 / page_tokens], n_layers, layer, kv_heads, kvh, page_tokens, v_dim) +
-                          key2 % page_tokens;
-            const float pk = ps[kk];
-#pragma unroll
-            for (int j = 0; j < BA_MAX_V_CHUNKS; ++j) {
-                const int d = lane + j * CELEG_WAVE;
-                if (d < v_dim) acc[j] = fmaf(pk, to_float(vp[static_cast<size_t>(d) * page_tokens]), acc[j]);
+        const int lo = phase == 0 ? 0 : first, hi = phase == 0 ? kept - 1 : pos;
+        for (int base = lo; base <= hi; base += CELEG_WAVE) {
+            const int key = base + lane;
+            float score = -INFINITY;
+            if (key <= hi) {
+                const T* kp = k_pool + ba_k_offset(pages[key / page_tokens], n_layers, layer, kv_heads, kvh, page_tokens,
+                                                   key % page_tokens, head_dim);
+                float dot = 0.f;
+                for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_float(kp[d]), dot);
+                score = dot * s;
+                if (r1) score -= b1 * logf(1.0f + b2 * static_cast<float>(pos - key));
             }
+            const float new_top = fmaxf(top, wave_max(score));     // (the round holds at least one visible key)
+            const float p = key <= hi ? expf(score - new_top) : 0.f;
+            const float keep = expf(top - new_top);                // 0 in the first round
+            total = total * keep + wave_sum(p);
+            top = new_top;
+            ps[lane] = p;
+            __syncthreads();
+            const int n_keys = min(CELEG_WAVE, hi - base + 1);
+#pragma unroll
+            for (int j = 0; j < BA_MAX_V_CHUNKS; ++j) acc[j] *= keep;
+            for (int kk = 0; kk < n_keys; ++kk) {
+                const int key2 = base + kk;
+                const T* vp = v_pool + ba_v_offset(pages[key2 / page_tokens], n_layers, layer, kv_heads, kvh, page_tokens, v_dim) +
+                              key2 % page_tokens;
+                const float pk = ps[kk];
+#pragma unroll
+                for (int j = 0; j < BA_MAX_V_CHUNKS; ++j) {
+                    const int d = lane + j * CELEG_WAVE;
+                    if (d < v_dim) acc[j] = fmaf(pk, to_float(vp[static_cast<size_t>(d) * page_tokens]), acc[j]);
+                }
+            }
+            __syncthreads();
         }
-        __syncthreads();
-    }
     }
     const float inv = 1.0f / total;
     T* orow = out + static_cast<size_t>(t) * ldo + static_cast<size_t>(h) * v_dim;
