@@ -212,7 +212,7 @@ def vabuzen_shape(width, heads, kv_heads, dim, window, l_dim, l_rot, rank, exper
     dense = {"kind": "dense", "ff": dense_ff}
     kinds = {"a": ("attention", attention), "l": ("latent_attention", latent)}
     layers = [{"type": kinds[c][0], "mixer": kinds[c][1], "mlp": moe if i % 2 else dense} for i, c in enumerate("allall")]
-    return {"architecture": "Vabuzen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.5, "logit_softcap": 30.0,
+    return {"architecture": "Vabuzen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7, "logit_softcap": 30.0,
             "loop": {"start": 1, "stop": 3, "times": 2}, "max_context": 8192, "layers": layers}
 
 

@@ -104,7 +104,7 @@ V3 = {"architecture": "Vabuzen", "vocab": 260, "width": 128, "norm": {"eps": 1e-
                  latent(8, 32, 32, 32, 64, 0.125, 10000.0, dense(64)),
                  attention(4, 2, 96, 128, 0.1, 4, (10000.0, 96), (16, 1), dense(96))]}
 # sizes that are multiples of two only: width, vocabulary, heads, ranks and feed-forwards that fill no tile or vector load
-V4 = {"architecture": "Vabuzen", "vocab": 333, "width": 100, "norm": {"eps": 1e-6}, "residual_mult": 0.5, "logit_softcap": 15.0,
+V4 = {"architecture": "Vabuzen", "vocab": 333, "width": 100, "norm": {"eps": 1e-6}, "residual_mult": 0.6, "logit_softcap": 12.0,
       "loop": {"start": 1, "stop": 2, "times": 2},
       "layers": [attention(3, 1, 20, 12, 0.22, 3, (10000.0, 10), (11, 2), dense(50)),
                  latent(3, 10, 6, 14, 18, 0.25, 777.0, moe(6, 2, 20, (3, 2), 2.0, 30)),
@@ -508,36 +508,6 @@ def test_window_attention_alone(tmp_path, taps, rot, mask):
     assert_close_f32(got, Wd["table"] + plain.window_attention(Wd["table"], Wd, "", m), "attention behind convolutions alone")
 
 
-def test_the_one_in_the_denominator_the_pairing_and_the_taps_show():
-    """The plain attention with an ordinary softmax, with the halves paired instead of neighbours, with
-    the taps in reverse order or with a window or a number of kept keys that is one off differs by far
-    more than any tolerance."""
-    t, m, _ = attention_case(60, 24, 2, 1, 16, 16, 0.5, 3, (100.0, 16), (9, 3))
-    Wd = doubles(t)
-    right = plain.window_attention(Wd["table"], Wd, "", m)
-
-    def moved(out):
-        return float((out - right).abs().max()) / float(right.abs().max())
-    n = 60
-    H, D = 2, 16
-    # an ordinary softmax: the same scores, weights that sum to one
-    q, k, v = (plain.causal_taps(Wd["table"] @ Wd[c].T, Wd[c + ".conv"]) for c in "qkv")
-    pos = torch.arange(n)
-    qh, kh = plain.rotate_neighbours(q.view(n, H, D), pos, 100.0, 16), plain.rotate_neighbours(k.view(n, 1, D), pos, 100.0, 16)
-    out = torch.zeros(n, H, D, dtype=torch.float64)
-    for i in range(n):
-        seen = [j for j in range(i + 1) if i - j < 9 or j < 3]
-        for a in range(H):
-            out[i, a] = torch.softmax((kh[seen, 0] @ qh[i, a]) * 0.5, 0) @ v.view(n, 1, D)[seen, 0]
-    assert moved(out.reshape(n, H * D) @ Wd["o"].T) > 0.1
-    flipped = dict(Wd, **{c + ".conv": Wd[c + ".conv"].flip(1) for c in "qkv"})
-    assert moved(plain.window_attention(Wd["table"], flipped, "", m)) > 0.1
-    for size, keep in ((8, 3), (10, 3), (9, 2), (9, 4)):
-        assert moved(plain.window_attention(Wd["table"], Wd, "", dict(m, mask={"size": size, "keep_first": keep}))) > 0.02, (size, keep)
-    halves = plain.rotate_halves(q.view(n, H, D), pos, 100.0, 16)
-    assert float((halves - qh).abs().max()) > 0.1 * float(qh.abs().max())
-
-
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_keys_at_the_windows_edge_and_kept_first_keys(tmp_path, dtype):
     """Rows whose weight sits on one key: the last key inside a window of 40 and the first one outside, the
@@ -701,23 +671,6 @@ def test_routed_experts_in_groups_alone(tmp_path, experts, top, groups, scale, s
     Wd = doubles(t)
     assert_close_f32(got, Wd["table"] + plain.routed_ff(Wd["table"], Wd, "", f), "routed experts alone")
     assert lm.paths()["routed_experts"] > 0
-
-
-def test_the_groups_the_renormalization_and_the_shared_expert_show():
-    """Without the groups other experts are chosen for many rows (the largest scores of a row often lie in a
-    group that loses); weights not divided by their sum, a factor left out or the shared expert left out move
-    the output by tens of percent."""
-    t, f, _ = experts_case(64, 40, 24, 12, 3, (4, 2), 2.0, 40)
-    Wd = doubles(t)
-    right = plain.routed_ff(Wd["table"], Wd, "", f)
-    score = torch.sigmoid(Wd["table"] @ Wd["router"].T)
-    differ = sum(sorted(plain.choose_experts(score[i], f["router"])[0]) != sorted(plain.choose_experts(score[i], {"experts": 12, "top": 3})[0])
-                 for i in range(64))
-    assert differ >= 16
-    moved = lambda out: float((out - right).abs().max()) / float(right.abs().max())
-    assert moved(plain.routed_ff(Wd["table"], Wd, "", dict(f, router=dict(f["router"], scale=1.0)))) > 0.1
-    assert moved(plain.routed_ff(Wd["table"], Wd, "", dict(f, shared=None))) > 0.1
-    assert moved(plain.routed_ff(Wd["table"], Wd, "", dict(f, router=dict(f["router"], groups={"count": 4, "keep": 1})))) > 0.1
 
 
 def test_dense_feed_forward_alone(tmp_path):
