@@ -1612,7 +1612,8 @@ private:
 };
 
 // ---------------------------------------------------------------------------- attention with a distance bias
-// Grouped-query softmax attention without a rotation: positions enter through the scores alone.
+// Grouped-query softmax attention whose options are parameters: positions enter through the scores (a factor on
+// the query, a distance bias) or, with a "position" part, through a rotation of q and k.
 //
 // q = W_q h, k = W_k h (head_dim a head), v = W_v h ("v_dim" a head, which may differ from head_dim).
 // score(i, j) = (q_i . k_j) * scale * f(i) - r1[h] ln(1 + r2[h] (i - j)) with
